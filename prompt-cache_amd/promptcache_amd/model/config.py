@@ -457,6 +457,174 @@ class DibizenShape:
                    logit_softcap=30.0, name=name)
 
 
+@dataclass
+class FivesunLayer:
+    """One layer of a Fivesun stack.  ``kind``: which mixer it has --
+
+    * ``"attention"``: softmax attention with ``heads`` query heads over ``kv_heads`` key/value heads (``dim`` query/key and
+      ``vdim`` value columns), per-head RMS norms on queries and keys, interleaved rotary positions on the first ``rot_dims``
+      columns (frequencies divided by ``rot_factor``), unit-RMS values, a learned sink per head in the softmax denominator, one
+      sigmoid output gate per head, keys visible only inside the query's own block of ``mask`` positions (0: all earlier keys);
+      ``v_mix``: the values are blended with those of the first such layer;
+    * ``"latent_attention"``: ``heads`` heads whose keys and values are up-projections of one cached latent of ``kv_rank``
+      columns per token, plus one rotated key part of ``rot_dim`` columns shared by all heads (YaRN-scaled frequencies:
+      ``rot_factor``, ``yarn_original``, ``yarn_fast``, ``yarn_slow``; ``yarn_original`` 0 = plain frequencies), a sliding window
+      of ``mask`` positions (0: none) and an element-wise sigmoid output gate;
+    * ``"mlstm"``: the matrix memory of xLSTM -- per head a ``dim`` x ``vdim`` state with exponential input gates, sigmoid forget
+      gates (pre-activations soft-capped at ``gate_cap``; 0 = not capped) and a running maximum that keeps the exponentials finite.
+
+    ``ff`` 0: no feed-forward; else a gated dense unit of that width, ``act`` its activation (relu, silu or gelu_tanh)."""
+    kind: str
+    heads: int = 0
+    kv_heads: int = 0
+    dim: int = 0
+    vdim: int = 0
+    scale: float = 1.0
+    mask: int = 0
+    rot_base: float = 10000.0
+    rot_dims: int = 0
+    rot_factor: float = 1.0
+    v_mix: bool = False
+    kv_rank: int = 0
+    rot_dim: int = 0
+    yarn_original: float = 0.0
+    yarn_fast: float = 32.0
+    yarn_slow: float = 1.0
+    gate_cap: float = 0.0
+    ff: int = 0
+    act: str = "relu"
+
+
+@dataclass
+class FivesunShape:
+    """Fivesun: decoder-only, a scaled embedding, layers in any order whose mixer is chunked softmax attention with sinks,
+    windowed latent attention or an mLSTM matrix memory, every sublayer between a norm before and a norm after it with a sigmoid
+    gate on its result (x <- x + norm_after(gate * f(norm_before(x)))), dense gated feed-forwards with biases.  Every size and
+    constant comes from ``config.json`` (``from_config``)."""
+    vocab_size: int
+    hidden_size: int
+    norm_eps: float
+    layers: list
+    embed_scale: float = 1.0
+    name: str = "fivesun"
+
+    ARCHITECTURE = "Fivesun"
+    KINDS = ("attention", "latent_attention", "mlstm")
+
+    @property
+    def num_hidden_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def first_v_mix(self) -> int:
+        """Index of the first layer whose values the later ``v_mix`` layers blend in (-1: none)."""
+        for i, l in enumerate(self.layers):
+            if l.kind == "attention" and l.v_mix:
+                return i
+        return -1
+
+    @classmethod
+    def from_config(cls, c: dict, name: str = "fivesun") -> "FivesunShape":
+        if c.get("architecture") != cls.ARCHITECTURE:
+            raise ValueError(f"config.json describes {c.get('architecture')!r}, not {cls.ARCHITECTURE}")
+        layers = []
+        for i, lc in enumerate(c["layers"]):
+            kind, m = lc.get("type"), lc.get("mixer") or {}
+            rot = m.get("rot") or {}
+            sc = rot.get("scaling") or {}
+            mask = int((m.get("mask") or {}).get("size") or 0)
+            if kind == "attention":
+                heads, dim = int(m["heads"]), int(m["dim"])
+                kv = int(m.get("kv_heads") or heads)
+                if heads % kv:
+                    raise ValueError(f"layer {i}: {heads} query heads do not divide over {kv} key heads")
+                lay = FivesunLayer(kind, heads=heads, kv_heads=kv, dim=dim, vdim=int(m.get("vdim") or dim),
+                                   scale=float(m.get("scale", dim ** -0.5)), mask=mask, rot_base=float(rot.get("base", 10000.0)),
+                                   rot_dims=int(rot.get("dims", dim if rot else 0)), rot_factor=float(sc.get("factor", 1.0)),
+                                   v_mix=bool(m.get("v_mix", False)))
+                if lay.rot_dims % 2 or lay.rot_dims > dim:
+                    raise ValueError(f"layer {i}: {lay.rot_dims} rotated columns of {dim}")
+            elif kind == "latent_attention":
+                heads, dim, rd = int(m["heads"]), int(m["dim"]), int(m.get("rot_dim") or 0)
+                lay = FivesunLayer(kind, heads=heads, kv_heads=1, dim=dim, vdim=int(m.get("vdim") or dim), kv_rank=int(m["kv_rank"]),
+                                   rot_dim=rd, rot_dims=rd, scale=float(m.get("scale", (dim + rd) ** -0.5)), mask=mask,
+                                   rot_base=float(rot.get("base", 10000.0)), rot_factor=float(sc.get("factor", 1.0)),
+                                   yarn_original=float(sc.get("original", 0.0)), yarn_fast=float(sc.get("fast", 32.0)),
+                                   yarn_slow=float(sc.get("slow", 1.0)))
+                if rd % 2 or int(rot.get("dims", rd)) != rd:
+                    raise ValueError(f"layer {i}: the rotated part has {rd} columns, the rotation {rot.get('dims')}")
+            elif kind == "mlstm":
+                heads, dim = int(m["heads"]), int(m["dim"])
+                lay = FivesunLayer(kind, heads=heads, kv_heads=heads, dim=dim, vdim=int(m.get("vdim") or dim),
+                                   gate_cap=float(m.get("gate_cap") or 0.0))
+            else:
+                raise ValueError(f"layer {i}: unknown mixer type {kind!r}")
+            mlp = lc.get("mlp")
+            if mlp:
+                if mlp.get("kind", "dense") != "dense":
+                    raise ValueError(f"layer {i}: unknown feed-forward kind {mlp.get('kind')!r}")
+                lay.ff = int(mlp["ff"])
+            layers.append(lay)
+        shape = cls(vocab_size=int(c["vocab"]), hidden_size=int(c["width"]), norm_eps=float((c.get("norm") or {}).get("eps", 1e-6)),
+                    layers=layers, embed_scale=float((c.get("embedding") or {}).get("scale", 1.0)), name=name)
+        shape.check()
+        return shape
+
+    def check(self) -> None:
+        first = self.first_v_mix
+        for i, l in enumerate(self.layers):
+            if l.kind not in self.KINDS:
+                raise ValueError(f"layer {i}: unknown mixer type {l.kind!r}")
+            if l.kind == "attention" and l.v_mix and (l.kv_heads, l.vdim) != (self.layers[first].kv_heads, self.layers[first].vdim):
+                raise ValueError(f"layer {i}: blends its values with layer {first}'s, which have another shape")
+
+    @classmethod
+    def from_dir(cls, path: str) -> "FivesunShape":
+        with open(os.path.join(path, "config.json")) as f:
+            return cls.from_config(json.load(f), name=os.path.basename(os.path.normpath(path)))
+
+    def to_config(self) -> dict:
+        """The ``config.json`` form (what ``from_config`` reads)."""
+        out = []
+        for l in self.layers:
+            if l.kind == "attention":
+                mixer = {"dim": l.dim, "heads": l.heads, "kv_heads": l.kv_heads, "scale": l.scale, "v_mix": l.v_mix, "vdim": l.vdim}
+                if l.rot_dims:
+                    mixer["rot"] = {"base": l.rot_base, "dims": l.rot_dims, "scaling": {"factor": l.rot_factor}}
+            elif l.kind == "latent_attention":
+                mixer = {"dim": l.dim, "heads": l.heads, "kv_rank": l.kv_rank, "rot_dim": l.rot_dim, "scale": l.scale, "vdim": l.vdim,
+                         "rot": {"base": l.rot_base, "dims": l.rot_dim}}
+                if l.yarn_original:
+                    mixer["rot"]["scaling"] = {"factor": l.rot_factor, "fast": l.yarn_fast, "original": l.yarn_original,
+                                               "slow": l.yarn_slow}
+            else:
+                mixer = {"dim": l.dim, "gate_cap": l.gate_cap, "heads": l.heads, "vdim": l.vdim}
+            if l.mask:
+                mixer["mask"] = {"size": l.mask}
+            out.append({"type": l.kind, "mixer": mixer, "mlp": {"ff": l.ff, "kind": "dense"} if l.ff else None})
+        return {"architecture": self.ARCHITECTURE, "embedding": {"scale": self.embed_scale}, "layers": out,
+                "norm": {"eps": self.norm_eps}, "vocab": self.vocab_size, "width": self.hidden_size}
+
+    @classmethod
+    def uniform(cls, vocab: int, width: int, pattern, heads: int, kv_heads: int, dim: int, ff: int, chunk: int = 0, window: int = 0,
+                kv_rank: int = 0, rot_dim: int = 64, name: str = "fivesun") -> "FivesunShape":
+        """A stack whose layers follow ``pattern`` (a sequence of mixer kinds), all with the same sizes and feed-forward."""
+        layers = []
+        for kind in pattern:
+            if kind == "attention":
+                lay = FivesunLayer(kind, heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, scale=dim ** -0.5, mask=chunk,
+                                   rot_base=500000.0, rot_dims=dim, rot_factor=2.0, v_mix=True)
+            elif kind == "latent_attention":
+                lay = FivesunLayer(kind, heads=heads, kv_heads=1, dim=dim, vdim=dim, kv_rank=kv_rank or 4 * dim, rot_dim=rot_dim,
+                                   rot_dims=rot_dim, scale=(dim + rot_dim) ** -0.5, mask=window, rot_base=250000.0, rot_factor=2.0,
+                                   yarn_original=2048.0)
+            else:
+                lay = FivesunLayer("mlstm", heads=heads, kv_heads=heads, dim=dim, vdim=dim, gate_cap=15.0)
+            lay.ff = ff
+            layers.append(lay)
+        return cls(vocab_size=vocab, hidden_size=width, norm_eps=1e-6, layers=layers, embed_scale=width ** 0.5, name=name)
+
+
 def architecture_of(path: str) -> str:
     """Which model family a checkpoint directory holds: ``architecture`` (Kazolorn) or HF's ``model_type``."""
     with open(os.path.join(path, "config.json")) as f:
@@ -465,4 +633,6 @@ def architecture_of(path: str) -> str:
         return "kazolorn"
     if c.get("architecture") == DibizenShape.ARCHITECTURE:
         return "dibizen"
+    if c.get("architecture") == FivesunShape.ARCHITECTURE:
+        return "fivesun"
     return str(c.get("model_type", "llama"))
