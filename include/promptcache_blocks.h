@@ -16,7 +16,7 @@
 extern "C" {
 #endif
 
-#define PCB_ABI_VERSION 2
+#define PCB_ABI_VERSION 3
 #define PCB_OK 0
 #define PCB_ERR_ARG (-2001)
 #define PCB_ERR_HIP_BASE (-3000)
@@ -30,6 +30,10 @@ const char* pcb_last_error_string(void);
 /* out[r][:] = fp32(table[ids[r]][:]) : the embedding rows as the first residual stream. */
 int pcb_embed_rows(const void* table, int32_t dtype, const int32_t* ids, float* out, int32_t n_rows, int32_t width, int32_t vocab,
                    void* stream);
+
+/* out[r][:] = scale * fp32(table[ids[r]][:]) : embedding rows times a constant (the product is taken in fp32). */
+int pcb_embed_scaled_rows(const void* table, int32_t dtype, const int32_t* ids, float scale, float* out, int32_t n_rows, int32_t width,
+                          int32_t vocab, void* stream);
 
 /* Weighted sum of residual streams + up to two RMS norms of the result, one workgroup per row:
  *   x[r]    = n_terms > 0 ? sum_j coef[j] * hist[j][src(r)] : hist[0][src(r)]       src(r) = rows ? rows[r] : r
@@ -60,7 +64,8 @@ int pcb_mix_norm(const pcb_mix_norm_args* a, void* stream);
  * groups    n_groups > 0: rows [group_off[g], group_off[g+1]) use W + g * w_group_stride (and W2 likewise); M is then an upper
  *           bound of group_off[n_groups] (the launch covers it; the kernel reads the offsets)
  * epilogue  PCB_EPI_STORE      v = acc + bias[n]
- *           PCB_EPI_SILU_MUL   v = silu(acc) * acc2, acc2 = A W2^T   (gated unit; no bias)
+ *           PCB_EPI_SILU_MUL   v = f(acc + bias[n]) * (acc2 + bias2[n]), acc2 = A W2^T   (gated unit; f = SiLU, or `act` when it is
+ *                              PCB_ACT_RELU / PCB_ACT_GELU_TANH / PCB_ACT_SILU; both biases optional)
  *           PCB_EPI_SCALE_ADD  v = (base ? base[m][n] : y32[m][n]) + col_scale[n] * (acc + bias[n]), stored fp32 (ldy)
  * output    STORE / SILU_MUL: element type E, or fp32 when out_f32; row m goes to y + (row_dst ? row_dst[m] : m) * ldy.
  *           split_n > 0 (STORE only): columns n >= split_n go to y2 instead: row m at y2 + row_off2[m], column c = n - split_n at
@@ -75,6 +80,8 @@ int pcb_mix_norm(const pcb_mix_norm_args* a, void* stream);
 #define PCB_ACT_RELU2 3
 #define PCB_ACT_SOFTPLUS 4
 #define PCB_ACT_SOFTCAP 5
+#define PCB_ACT_RELU 6      /* max(z, 0) */
+#define PCB_ACT_GELU_TANH 7 /* 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))) */
 typedef struct pcb_linear_args {
     uint32_t struct_bytes;
     int32_t dtype;
@@ -113,6 +120,7 @@ typedef struct pcb_linear_args {
     int32_t act_split; /* > 0: columns n >= act_split take act2 instead of act */
     int32_t act2;
     float act_param;   /* PCB_ACT_SOFTCAP: the cap */
+    const void* bias2; /* [N] E, may be null: the second product's bias of the gated epilogue */
 } pcb_linear_args;
 int pcb_linear(const pcb_linear_args* a, void* stream);
 
@@ -212,10 +220,12 @@ typedef struct pcb_hyper_norm_args {
 } pcb_hyper_norm_args;
 int pcb_hyper_norm(const pcb_hyper_norm_args* a, void* stream);
 
-/* out[r][c] = E( (gain ? x[r][c] / sqrt(mean_c x[r]^2 + eps) * gain[c] : x[r][c]) * (gate ? gate[r][c] : 1) ), x fp32 [n_rows][ldx],
- * gate E [n_rows][ldg], out E [n_rows][ldo]: a unit norm over all heads' outputs with an element-wise gate. */
+/* out[r][c] = E( (gain ? x[r][c] / sqrt(mean x[r]^2 + eps) * gain[c] : x[r][c]) * (gate ? gate[r][c] : 1) ), x fp32 [n_rows][ldx],
+ * gate E [n_rows][ldg], out E [n_rows][ldo]: a unit norm with an element-wise gate.  The mean runs over all `cols` columns
+ * (group_cols <= 0: one norm over all heads' outputs) or over each run of group_cols columns by itself (a norm per head;
+ * group_cols divides cols; then the norm is taken with or without a gain). */
 int pcb_gated_norm(const float* x, int64_t ldx, const float* gain, const void* gate, int64_t ldg, void* out, int64_t ldo,
-                   int32_t dtype, float eps, int32_t n_rows, int32_t cols, void* stream);
+                   int32_t dtype, float eps, int32_t n_rows, int32_t cols, int32_t group_cols, void* stream);
 
 /* Router choice over n_out outputs per row (logits fp32 [n_rows][n_out]):
  *   score s = score_fn == PCB_SCORE_SOFTMAX ? softmax(logits) : sigmoid(logits);  choice score = s + correction (if given)
@@ -243,8 +253,11 @@ int pcb_moe_mix(const float* pair_out, const int32_t* expert, const float* weigh
  * interleave in one plane), or column by column (v_cols = 1: column c of key j at vcache + s * v_slot_stride + g * v_head_stride +
  * c * v_stride + j; every column must be readable up to the next multiple of 32 keys, and v_stride a multiple of 8), which lets
  * the value operand of the matrix cores be read with wide loads.  The cache already holds the queries' own keys and values.  score = q_scale[row] * scale * q.k (q_scale null: 1); key j is seen by the query at position i iff j <= i and
- * (window <= 0 or i - j < window).  The result (E [rows][ldo], head h at column h * vdim) is multiplied element-wise by
- * gate[row][..] (E, ldg) when given.  dim, vdim <= 256. */
+ * (window <= 0 or i - j < window) and (block <= 0 or floor(i / block) == floor(j / block): blocks of positions counted from 0, a
+ * key is seen inside the query's own block only).  sink (fp32 [H], optional): the softmax denominator of head h also holds
+ * exp(sink[h]) -- a term without key or value, not scaled.  The result (E [rows][ldo], head h at column h * vdim) is multiplied by
+ * a gate when given (E, row stride ldg): element-wise gate[row][h * vdim + c], or one number per head gate[row][h] when
+ * gate_per_head.  dim <= 384, vdim <= 256. */
 typedef struct pcb_attn_softmax_args {
     uint32_t struct_bytes;
     int32_t dtype;
@@ -269,6 +282,9 @@ typedef struct pcb_attn_softmax_args {
                          leave (maximum, denominator, weighted values) in `part`; a second launch merges them.  For steps of few
                          rows over long caches. */
     float* part;      /* fp32 [rows][H][n_splits][vdim + 2], rows = the flat rows the tiles cover (row index = flat row) */
+    int32_t block;
+    const float* sink;
+    int32_t gate_per_head;
 } pcb_attn_softmax_args;
 int pcb_attn_softmax(const pcb_attn_softmax_args* a, void* stream);
 
@@ -349,6 +365,101 @@ int pcb_selective_scan(const pcb_selective_scan_args* a, void* stream);
  * local, start: fp32 [segments][elems]; coef fp32 [elems]; x fp32 [segments][elems / group]. */
 int pcb_state_chain(const float* local, float* start, float* state, int64_t slot_stride, const int32_t* chains, int32_t n_chains,
                     const float* coef, const float* x, int32_t elems, int32_t group, void* stream);
+
+/* ---- sublayers between two norms, per-head preparation of queries / keys / values, matrix memories ------------------------------ */
+
+/* A residual step with a norm after the sublayer and the norm before the next one, one workgroup per row, in two optional halves:
+ *   write (y given):  t = y[src] * (gate ? gate[src] : 1);  x[src] += post_gain ? t / sqrt(mean(t^2) + eps) * post_gain : t
+ *                     (with `rows` the sum is used but not written back)
+ *   read (out given): out[r] = x[src] / sqrt(mean(x[src]^2) + eps) * gain as E;  x_out[r] = x[src] (fp32) if given
+ * src = rows ? rows[r] : r.  y fp32 [..][width]; gate E rows of stride ldg; x fp32 [..][width].  width <= 16384. */
+typedef struct pcb_post_norm_args {
+    uint32_t struct_bytes;
+    int32_t dtype;
+    float* x;
+    const float* y;
+    const void* gate;
+    int64_t ldg;
+    const float* post_gain;
+    const float* gain;
+    void* out;
+    float* x_out;
+    const int32_t* rows;
+    float eps;
+    int32_t n_rows;
+    int32_t width;
+} pcb_post_norm_args;
+int pcb_post_norm(const pcb_post_norm_args* a, void* stream);
+
+/* Per-head preparation of projected rows: up to four segments (queries, keys, values, ...) of one launch, each `heads` heads of
+ * head_dim columns read from E rows (src + row * ld_src + h * src_head_stride).  Per head, in this order, all in fp32:
+ *   norm:   x <- x / sqrt(mean(x^2) + eps)  (norm != 0), times gain[c] when given
+ *   blend:  x <- (1 - blend[0]) x + blend[0] * other[row][h * head_dim + c]      (other fp32, blend one float on the device)
+ *   keep:   keep[row][h * head_dim + c] = x                                       (fp32: what a later launch blends with)
+ *   rotate: columns rot_off + 2i, rot_off + 2i + 1 (i < rot_dims / 2) turn by the angle pos[row] * freqs[i]:
+ *           (u, v) <- rot_mag * (u cos - v sin, v cos + u sin); the angle is a float64 product, other columns pass unchanged
+ *   store:  E at dst + (row_off ? row_off[row] : row * ld_dst) + h * head_stride + c * col_stride  (rows of a matrix, a cache kept
+ *           row by row, or one kept column by column)
+ * freqs: float64 [rot_dims / 2] on the device, shared by the segments that rotate (they have the same rot_dims).  head_dim <= 1024. */
+typedef struct pcb_head_prep_seg {
+    const void* src;
+    int64_t ld_src;
+    int64_t src_head_stride;
+    int32_t heads, head_dim;
+    int32_t norm;
+    const float* gain;
+    const float* blend;
+    const float* other;
+    int64_t ld_other;
+    float* keep;
+    int64_t ld_keep;
+    int32_t rot_off, rot_dims;
+    void* dst;
+    int64_t ld_dst;
+    const int64_t* row_off;
+    int64_t head_stride, col_stride;
+} pcb_head_prep_seg;
+typedef struct pcb_head_prep_args {
+    uint32_t struct_bytes;
+    int32_t dtype;
+    int32_t n_rows;
+    int32_t n_segs;
+    const int32_t* pos;
+    const double* freqs;
+    float rot_mag;
+    float eps;
+    pcb_head_prep_seg seg[4];
+} pcb_head_prep_args;
+int pcb_head_prep(const pcb_head_prep_args* a, void* stream);
+
+/* Matrix memory with exponential gating (mLSTM): per (slot, head) a state S [dim][vdim], a normaliser n [dim] and a running
+ * maximum m, all fp32, zero before position 0.  Per token, with the head's log input gate li and log forget gate lf:
+ *   li = cap(gi),  lf = logsigmoid(cap(gf)),  cap(z) = gate_cap > 0 ? gate_cap tanh(z / gate_cap) : z
+ *   m' = max(lf + m, li);  S' = exp(lf + m - m') S + exp(li - m') k v^T;  n' = exp(lf + m - m') n + exp(li - m') k
+ *   o = S'^T (q_scale q) / (max(|n' . q_scale q|, exp(-m')) + 1e-6)
+ * q, k: E rows, head h at column h * dim; v: head h at column h * vdim; gi, gf: E rows, one column per head (the gates'
+ * pre-activations, bias included); out fp32 [rows][ldo].  request r = {slot, first position, tokens, first flat row} as in
+ * pcb_decay_attn.  state: fp32 per slot [H][dim * vdim + dim + 1] (S, then n, then m), slot_stride floats apart. */
+typedef struct pcb_mlstm_args {
+    uint32_t struct_bytes;
+    int32_t dtype;
+    const void* q;
+    const void* k;
+    const void* v;
+    const void* gi;
+    const void* gf;
+    int64_t ldq, ldk, ldv, ldgi, ldgf;
+    const int32_t* reqs;
+    int32_t n_reqs;
+    float* state;
+    int64_t slot_stride;
+    int32_t H, dim, vdim;
+    float q_scale;
+    float gate_cap;
+    float* out;
+    int64_t ldo;
+} pcb_mlstm_args;
+int pcb_mlstm(const pcb_mlstm_args* a, void* stream);
 
 #ifdef __cplusplus
 }

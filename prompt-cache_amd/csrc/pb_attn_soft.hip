@@ -1,5 +1,6 @@
 // pcb_attn_softmax: causal softmax attention over a slot-addressed cache with separate keys and values (grouped key/value
-// heads, value size independent of the key size, optional sliding window, per-row score factor, optional output gate).
+// heads, value size independent of the key size, optional sliding window or blocks of positions that see only themselves, per-row
+// score factor, optional learned sink in the denominator, optional output gate per element or per head).
 //
 // One workgroup = one tile of up to 16 queries x one query head; its four waves take every fourth block of 32 keys and keep a
 // running maximum / denominator per query (online softmax), then merge through LDS.  Both products are "swapped" so that no
@@ -129,6 +130,9 @@ __global__ __launch_bounds__(64 * AW) void attn_softmax_kernel(pcb_attn_softmax_
     // scores are kept in units of ln 2 (the factor log2(e) rides on the scale), so that every exponential is one v_exp_f32
     const float sc = a.scale * (a.q_scale ? a.q_scale[qrow] : 1.0f) * 1.44269504088896f;
     const float NEG = -__builtin_inff();
+    // the oldest key this lane's query sees: the window's and the block's edges, whichever is later
+    int key_lo = a.window > 0 ? qpos - a.window + 1 : 0;
+    if (a.block > 0) key_lo = max(key_lo, qpos / a.block * a.block);
 
     float m = NEG, l = 0.0f;
     f4 o[VB];
@@ -136,6 +140,7 @@ __global__ __launch_bounds__(64 * AW) void attn_softmax_kernel(pcb_attn_softmax_
     for (int vb = 0; vb < VB; ++vb) o[vb] = f4{0.f, 0.f, 0.f, 0.f};
 
     int kb_lo = a.window > 0 ? (pos0 - a.window + 1 > 0 ? (pos0 - a.window + 1) / 32 : 0) : 0;
+    if (a.block > 0) kb_lo = max(kb_lo, pos0 / a.block * a.block / 32);      // (the tile's first query has the oldest block)
     int kb_hi = last / 32;
     if (a.n_splits > 1) {                                   // this workgroup's run of the key blocks (it may be empty)
         const int per = (kb_hi - kb_lo + a.n_splits) / a.n_splits;
@@ -179,7 +184,7 @@ __global__ __launch_bounds__(64 * AW) void attn_softmax_kernel(pcb_attn_softmax_
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int key = kb * 32 + kt * 16 + 4 * g + r;
-                const bool seen = key <= qpos && (a.window <= 0 || qpos - key < a.window);
+                const bool seen = key <= qpos && key >= key_lo;
                 s[kt * 4 + r] = seen ? acc[r] * sc : NEG;
             }
         }
@@ -278,17 +283,27 @@ __global__ __launch_bounds__(64 * AW) void attn_softmax_kernel(pcb_attn_softmax_
             }
         return;
     }
-    const float inv = 1.0f / lt;
+    float keep = 1.0f;
+    if (a.sink) {
+        // one more term exp(sink) without a value: the sum moves to the larger of the two maxima (a query always sees itself, so
+        // m_use is a number)
+        const float sk = a.sink[h] * 1.44269504088896f;
+        const float top = fmaxf(m_use, sk);
+        keep = __builtin_amdgcn_exp2f(m_use - top);
+        lt = lt * keep + __builtin_amdgcn_exp2f(sk - top);
+    }
+    const float inv = keep / lt;
     E* op = (E*)a.out + qrow * a.ldo + (int64_t)h * vdim;
-    const E* gp = a.gate ? (const E*)a.gate + qrow * a.ldg + (int64_t)h * vdim : nullptr;
+    const E* gp = a.gate ? (const E*)a.gate + qrow * a.ldg + (a.gate_per_head ? 0 : (int64_t)h * vdim) : nullptr;
+    const float gh = (gp && a.gate_per_head) ? to_f32(gp[h]) : 1.0f;
 #pragma unroll
     for (int vb = 0; vb < VB; ++vb)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int col = vb * 16 + 4 * g + r;
             if (col < vdim) {
-                float v = o[vb][r] * inv;
-                if (gp) v *= to_f32(gp[col]);
+                float v = o[vb][r] * inv * gh;
+                if (gp && !a.gate_per_head) v *= to_f32(gp[col]);
                 op[col] = from_f32<E>(v);
             }
         }
@@ -313,8 +328,15 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(pcb_attn_softmax_args a
             l += f * pp[z * (vdim + 2) + vdim + 1];
             o += f * pp[z * (vdim + 2) + col];
         }
+        if (a.sink) {
+            const float sk = a.sink[h] * 1.44269504088896f;
+            const float top = fmaxf(m_use, sk);
+            const float keep = __builtin_amdgcn_exp2f(m_use - top);
+            l = l * keep + __builtin_amdgcn_exp2f(sk - top);
+            o *= keep;
+        }
         float v = o / l;
-        if (a.gate) v *= to_f32(((const E*)a.gate)[qrow * a.ldg + (int64_t)h * vdim + col]);
+        if (a.gate) v *= to_f32(((const E*)a.gate)[qrow * a.ldg + (a.gate_per_head ? (int64_t)h : (int64_t)h * vdim + col)]);
         ((E*)a.out)[qrow * a.ldo + (int64_t)h * vdim + col] = from_f32<E>(v);
     }
 }
@@ -327,8 +349,10 @@ int dispatch(const pcb_attn_softmax_args& a, hipStream_t stream) {
         hipLaunchKernelGGL((attn_softmax_kernel<E, 2, 4>), grid, block, 0, stream, a);
     else if (big <= 128)
         hipLaunchKernelGGL((attn_softmax_kernel<E, 4, 8>), grid, block, 0, stream, a);
-    else
+    else if (a.dim <= 256)
         hipLaunchKernelGGL((attn_softmax_kernel<E, 8, 16>), grid, block, 0, stream, a);
+    else
+        hipLaunchKernelGGL((attn_softmax_kernel<E, 12, 16>), grid, block, 0, stream, a);
     if (a.n_splits > 1) hipLaunchKernelGGL(attn_merge_kernel<E>, dim3(a.n_tiles, a.H), dim3(256), 0, stream, a);
     return pcb_check_launch("attn_softmax_kernel");
 }
@@ -338,15 +362,16 @@ int dispatch(const pcb_attn_softmax_args& a, hipStream_t stream) {
 PCB_EXPORT int pcb_attn_softmax(const pcb_attn_softmax_args* a, void* stream) {
     PCB_REQUIRE(a && a->struct_bytes == sizeof(pcb_attn_softmax_args), PCB_ERR_ARG, "pcb_attn_softmax: struct size mismatch");
     PCB_REQUIRE(a->dtype == PCB_BF16 || a->dtype == PCB_F32, PCB_ERR_ARG, "pcb_attn_softmax: unknown dtype");
-    PCB_REQUIRE(a->n_tiles >= 0 && a->H > 0 && a->Hkv > 0 && a->H % a->Hkv == 0 && a->dim > 0 && a->dim <= 256 && a->vdim > 0 &&
+    PCB_REQUIRE(a->n_tiles >= 0 && a->H > 0 && a->Hkv > 0 && a->H % a->Hkv == 0 && a->dim > 0 && a->dim <= 384 && a->vdim > 0 &&
                     a->vdim <= 256 && a->ldq >= (int64_t)a->H * a->dim && a->ldo >= (int64_t)a->H * a->vdim &&
                     a->row_stride >= a->dim && (a->v_cols ? (a->v_stride % 8 == 0 && a->v_stride > 0 && (uintptr_t)a->vcache % 16 == 0 &&
                                                              a->v_head_stride % 8 == 0 && a->v_slot_stride % 8 == 0)
                                                           : a->v_stride >= a->vdim),
-                PCB_ERR_ARG, "pcb_attn_softmax: bad sizes (key and value sizes up to 256; a column-wise value cache in multiples of 8)");
+                PCB_ERR_ARG, "pcb_attn_softmax: bad sizes (key size up to 384, value size up to 256; a column-wise value cache in multiples of 8)");
     if (a->n_tiles == 0) return PCB_OK;
-    PCB_REQUIRE(a->q && a->tiles && a->kcache && a->vcache && a->out && (!a->gate || a->ldg >= (int64_t)a->H * a->vdim), PCB_ERR_ARG,
-                "pcb_attn_softmax: null pointer");
+    PCB_REQUIRE(a->q && a->tiles && a->kcache && a->vcache && a->out &&
+                    (!a->gate || a->ldg >= (a->gate_per_head ? (int64_t)a->H : (int64_t)a->H * a->vdim)),
+                PCB_ERR_ARG, "pcb_attn_softmax: null pointer");
     PCB_REQUIRE(a->n_splits <= 1 || (a->part && a->n_splits <= 64), PCB_ERR_ARG, "pcb_attn_softmax: up to 64 runs, with their scratch");
     return a->dtype == PCB_BF16 ? dispatch<pcb::bf16_t>(*a, (hipStream_t)stream) : dispatch<float>(*a, (hipStream_t)stream);
 }

@@ -51,18 +51,20 @@ __device__ __forceinline__ float apply_act(int act, float v, float param) {
         case PCB_ACT_RELU2: return v > 0.0f ? v * v : 0.0f;
         case PCB_ACT_SOFTPLUS: return v > 20.0f ? v : log1pf(expf(v));
         case PCB_ACT_SOFTCAP: return param * tanhf(v / param);
+        case PCB_ACT_RELU: return v > 0.0f ? v : 0.0f;
+        case PCB_ACT_GELU_TANH: return 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
         default: return v;
     }
 }
 
 // one result element through the epilogue (see pcb_linear_args)
 template <typename E, int EPI>
-__device__ __forceinline__ void emit(const pcb_linear_args& a, int m, int n, float acc, float acc2, float bv, float cs) {
+__device__ __forceinline__ void emit(const pcb_linear_args& a, int m, int n, float acc, float acc2, float bv, float cs, float bv2 = 0.0f) {
     float v = acc + bv;
     if (EPI == PCB_EPI_STORE && (a.act | a.act2) && !(a.split_n > 0 && n >= a.split_n) && !(a.split_n3 > 0 && n >= a.split_n3))
         // (the split-off parts are stored as they are)
         v = apply_act((a.act_split > 0 && n >= a.act_split) ? a.act2 : a.act, v, a.act_param);
-    if (EPI == PCB_EPI_SILU_MUL) v = acc / (1.0f + expf(-acc)) * acc2;
+    if (EPI == PCB_EPI_SILU_MUL) v = apply_act(a.act == PCB_ACT_NONE ? PCB_ACT_SILU : a.act, v, 0.0f) * (acc2 + bv2);
     if (EPI == PCB_EPI_SCALE_ADD) {
         float* y = (float*)a.y + (int64_t)m * a.ldy + n;
         const float b0 = a.base ? a.base[(int64_t)m * a.ldbase + n] : *y;
@@ -211,13 +213,14 @@ __global__ __launch_bounds__(256) void linear_kernel(pcb_linear_args a) {
         const int n = n_lo + (wn * TN + j) * 16 + l15;
         if (n >= N) continue;
         const float bv = bias ? to_f32(bias[n]) : 0.0f;
+        const float bv2 = (TWO && a.bias2) ? to_f32(((const E*)a.bias2)[n]) : 0.0f;
         const float cs = (EPI == PCB_EPI_SCALE_ADD) ? a.col_scale[n] : 0.0f;
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int m = m_lo + (wm * TM + i) * 16 + 4 * group + r;
-                if (m < m_hi) emit<E, EPI>(a, m, n, acc[i][j][r], TWO ? acc2[i][j][r] : 0.0f, bv, cs);
+                if (m < m_hi) emit<E, EPI>(a, m, n, acc[i][j][r], TWO ? acc2[i][j][r] : 0.0f, bv, cs, bv2);
             }
     }
 }
@@ -313,11 +316,12 @@ __global__ __launch_bounds__(64 * SKW) void linear_skinny_kernel(pcb_linear_args
     if (n >= N) return;
     const E* bias = (const E*)a.bias;
     const float bv = bias ? to_f32(bias[n]) : 0.0f;
+    const float bv2 = (TWO && a.bias2) ? to_f32(((const E*)a.bias2)[n]) : 0.0f;
     const float cs = (EPI == PCB_EPI_SCALE_ADD) ? a.col_scale[n] : 0.0f;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const int m = m_lo + 4 * group + r;
-        if (m < m_hi) emit<E, EPI>(a, m, n, acc[r], acc2[r], bv, cs);
+        if (m < m_hi) emit<E, EPI>(a, m, n, acc[r], acc2[r], bv, cs, bv2);
     }
 }
 
@@ -365,15 +369,19 @@ PCB_EXPORT int pcb_linear(const pcb_linear_args* a, void* stream) {
     PCB_REQUIRE(a->dtype == PCB_BF16 || a->dtype == PCB_F32, PCB_ERR_ARG, "pcb_linear: unknown dtype");
     PCB_REQUIRE(a->M >= 0 && a->N > 0 && a->K > 0 && a->ldx >= a->K && a->ldw >= a->K, PCB_ERR_ARG, "pcb_linear: bad sizes");
     PCB_REQUIRE(a->epilogue >= PCB_EPI_STORE && a->epilogue <= PCB_EPI_SCALE_ADD, PCB_ERR_ARG, "pcb_linear: unknown epilogue");
-    PCB_REQUIRE(a->act >= PCB_ACT_NONE && a->act <= PCB_ACT_SOFTCAP && a->act2 >= PCB_ACT_NONE && a->act2 <= PCB_ACT_SOFTCAP &&
-                    a->act_split >= 0 && ((a->act | a->act2) == 0 || a->epilogue == PCB_EPI_STORE),
-                PCB_ERR_ARG, "pcb_linear: an activation goes with the plain store epilogue");
+    PCB_REQUIRE(a->act >= PCB_ACT_NONE && a->act <= PCB_ACT_GELU_TANH && a->act2 >= PCB_ACT_NONE && a->act2 <= PCB_ACT_GELU_TANH &&
+                    a->act_split >= 0 &&
+                    ((a->act | a->act2) == 0 || a->epilogue == PCB_EPI_STORE ||
+                     (a->epilogue == PCB_EPI_SILU_MUL && a->act2 == 0 &&
+                      (a->act == PCB_ACT_SILU || a->act == PCB_ACT_RELU || a->act == PCB_ACT_GELU_TANH))),
+                PCB_ERR_ARG, "pcb_linear: an activation goes with the plain store epilogue (the gated one takes silu, relu or gelu_tanh)");
     PCB_REQUIRE((a->act != PCB_ACT_SOFTCAP && a->act2 != PCB_ACT_SOFTCAP) || a->act_param > 0.0f, PCB_ERR_ARG,
                 "pcb_linear: the soft cap must be positive");
     if (a->M == 0) return PCB_OK;
     PCB_REQUIRE(a->x && a->w && a->y, PCB_ERR_ARG, "pcb_linear: null pointer");
     PCB_REQUIRE(a->n_groups >= 0 && (a->n_groups == 0 || a->group_off), PCB_ERR_ARG, "pcb_linear: groups need their offsets");
-    PCB_REQUIRE(a->epilogue != PCB_EPI_SILU_MUL || (a->w2 && !a->bias), PCB_ERR_ARG, "pcb_linear: the gated epilogue takes w2 and no bias");
+    PCB_REQUIRE(a->epilogue != PCB_EPI_SILU_MUL || a->w2, PCB_ERR_ARG, "pcb_linear: the gated epilogue takes w2");
+    PCB_REQUIRE(a->epilogue == PCB_EPI_SILU_MUL || !a->bias2, PCB_ERR_ARG, "pcb_linear: a second bias goes with the gated epilogue");
     PCB_REQUIRE(a->epilogue != PCB_EPI_SCALE_ADD || (a->col_scale && a->ldy >= a->N && !a->row_dst), PCB_ERR_ARG,
                 "pcb_linear: scale-add needs col_scale and a plain fp32 destination");
     PCB_REQUIRE(a->split_n == 0 || (a->epilogue == PCB_EPI_STORE && a->split_n > 0 && a->split_n < a->N && a->y2 && a->row_off2 &&

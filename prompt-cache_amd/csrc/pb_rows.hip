@@ -42,12 +42,12 @@ __device__ __forceinline__ void block_sum(float (&v)[NV], float* red) {
 
 template <typename E>
 __global__ __launch_bounds__(256) void embed_rows_kernel(const E* __restrict__ table, const int32_t* __restrict__ ids,
-                                                         float* __restrict__ out, int width, int vocab) {
+                                                         float* __restrict__ out, int width, int vocab, float scale = 1.0f) {
     const int r = blockIdx.x;
     int id = ids[r];
     id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
     const E* src = table + (int64_t)id * width;
-    for (int c = threadIdx.x; c < width; c += 256) out[(int64_t)r * width + c] = to_f32(src[c]);
+    for (int c = threadIdx.x; c < width; c += 256) out[(int64_t)r * width + c] = scale * to_f32(src[c]);
 }
 
 // one workgroup per output row; the row is held in LDS between the sum and the norms (width * 4 bytes of dynamic LDS)
@@ -192,10 +192,24 @@ PCB_EXPORT int pcb_embed_rows(const void* table, int32_t dtype, const int32_t* i
     PCB_REQUIRE(table && ids && out, PCB_ERR_ARG, "pcb_embed_rows: null pointer");
     if (dtype == PCB_BF16)
         hipLaunchKernelGGL(embed_rows_kernel<bf16_t>, dim3(n_rows), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)table, ids, out,
-                           width, vocab);
+                           width, vocab, 1.0f);
     else
         hipLaunchKernelGGL(embed_rows_kernel<float>, dim3(n_rows), dim3(256), 0, (hipStream_t)stream, (const float*)table, ids, out,
-                           width, vocab);
+                           width, vocab, 1.0f);
+    return pcb_check_launch("embed_rows_kernel");
+}
+
+PCB_EXPORT int pcb_embed_scaled_rows(const void* table, int32_t dtype, const int32_t* ids, float scale, float* out, int32_t n_rows,
+                                     int32_t width, int32_t vocab, void* stream) {
+    PCB_REQUIRE(PCB_DTYPE_OK(dtype) && n_rows >= 0 && width > 0 && vocab > 0, PCB_ERR_ARG, "pcb_embed_scaled_rows: bad sizes");
+    if (n_rows == 0) return PCB_OK;
+    PCB_REQUIRE(table && ids && out, PCB_ERR_ARG, "pcb_embed_scaled_rows: null pointer");
+    if (dtype == PCB_BF16)
+        hipLaunchKernelGGL(embed_rows_kernel<bf16_t>, dim3(n_rows), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)table, ids, out,
+                           width, vocab, scale);
+    else
+        hipLaunchKernelGGL(embed_rows_kernel<float>, dim3(n_rows), dim3(256), 0, (hipStream_t)stream, (const float*)table, ids, out,
+                           width, vocab, scale);
     return pcb_check_launch("embed_rows_kernel");
 }
 
@@ -374,6 +388,77 @@ __global__ __launch_bounds__(256) void gated_norm_kernel(const float* __restrict
     }
 }
 
+// the same with a norm per run of `group` columns (a head): one wave per (row, group) pair, four pairs per workgroup
+template <typename E>
+__global__ __launch_bounds__(256) void gated_group_norm_kernel(const float* __restrict__ x, int64_t ldx, const float* __restrict__ gain,
+                                                               const E* __restrict__ gate, int64_t ldg, E* __restrict__ out, int64_t ldo,
+                                                               float eps, int cols, int group, int64_t n_pairs) {
+    const int lane = threadIdx.x & 63;
+    const int64_t pair = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (pair >= n_pairs) return;
+    const int per = cols / group;
+    const int64_t r = pair / per;
+    const int c0 = (int)(pair % per) * group;
+    float ss = 0.0f;
+    for (int c = lane; c < group; c += 64) {
+        const float v = x[r * ldx + c0 + c];
+        ss += v * v;
+    }
+    ss = wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)group + eps);
+    for (int c = lane; c < group; c += 64) {
+        float v = x[r * ldx + c0 + c] * inv;
+        if (gain) v *= gain[c0 + c];
+        if (gate) v *= to_f32(gate[r * ldg + c0 + c]);
+        out[r * ldo + c0 + c] = from_f32<E>(v);
+    }
+}
+
+// one workgroup per row; the row waits in LDS between the two sums (width * 4 bytes of dynamic LDS)
+template <typename E>
+__global__ __launch_bounds__(1024) void post_norm_kernel(pcb_post_norm_args a) {
+    extern __shared__ float row[];
+    __shared__ float red[16];
+    const int r = blockIdx.x, W = a.width;
+    const int64_t src = a.rows ? a.rows[r] : r;
+    float* __restrict__ x = a.x + src * W;
+    float ss[1] = {0.0f};
+    if (a.y) {
+        const float* __restrict__ y = a.y + src * W;
+        const E* __restrict__ g = a.gate ? (const E*)a.gate + src * a.ldg : nullptr;
+        for (int c = threadIdx.x; c < W; c += blockDim.x) {
+            const float t = y[c] * (g ? to_f32(g[c]) : 1.0f);
+            row[c] = t;
+            ss[0] += t * t;
+        }
+        float inv = 1.0f;
+        if (a.post_gain) {
+            block_sum<1>(ss, red);
+            inv = 1.0f / sqrtf(ss[0] / (float)W + a.eps);
+        }
+        ss[0] = 0.0f;
+        for (int c = threadIdx.x; c < W; c += blockDim.x) {          // (a thread meets its own columns again: no barrier needed)
+            const float v = x[c] + (a.post_gain ? row[c] * inv * a.post_gain[c] : row[c]);
+            row[c] = v;
+            if (!a.rows) x[c] = v;
+            ss[0] += v * v;
+        }
+    } else {
+        for (int c = threadIdx.x; c < W; c += blockDim.x) {
+            const float v = x[c];
+            row[c] = v;
+            ss[0] += v * v;
+        }
+    }
+    if (a.x_out)
+        for (int c = threadIdx.x; c < W; c += blockDim.x) a.x_out[(int64_t)r * W + c] = row[c];
+    if (!a.out) return;
+    block_sum<1>(ss, red);
+    const float inv = 1.0f / sqrtf(ss[0] / (float)W + a.eps);
+    E* o = (E*)a.out + (int64_t)r * W;
+    for (int c = threadIdx.x; c < W; c += blockDim.x) o[c] = from_f32<E>(row[c] * inv * a.gain[c]);
+}
+
 // one wave per row: scores and choice scores in LDS, group maxima by lanes, then rounds of a wave-wide arg-max
 __global__ __launch_bounds__(256) void router_select_kernel(const float* __restrict__ logits, int n_rows, int n_out, int top, int score_fn,
                                                             const float* __restrict__ correction, int groups, int keep, int renorm,
@@ -517,11 +602,23 @@ PCB_EXPORT int pcb_hyper_norm(const pcb_hyper_norm_args* a, void* stream) {
 }
 
 PCB_EXPORT int pcb_gated_norm(const float* x, int64_t ldx, const float* gain, const void* gate, int64_t ldg, void* out, int64_t ldo,
-                              int32_t dtype, float eps, int32_t n_rows, int32_t cols, void* stream) {
+                              int32_t dtype, float eps, int32_t n_rows, int32_t cols, int32_t group_cols, void* stream) {
     PCB_REQUIRE(PCB_DTYPE_OK(dtype) && n_rows >= 0 && cols > 0 && ldx >= cols && ldo >= cols && (!gate || ldg >= cols), PCB_ERR_ARG,
                 "pcb_gated_norm: bad sizes");
+    PCB_REQUIRE(group_cols <= 0 || cols % group_cols == 0, PCB_ERR_ARG, "pcb_gated_norm: the groups must divide the columns");
     if (n_rows == 0) return PCB_OK;
     PCB_REQUIRE(x && out, PCB_ERR_ARG, "pcb_gated_norm: null pointer");
+    if (group_cols > 0 && group_cols < cols) {
+        const int64_t pairs = (int64_t)n_rows * (cols / group_cols);
+        const dim3 grid((unsigned)((pairs + 3) / 4));
+        if (dtype == PCB_BF16)
+            hipLaunchKernelGGL(gated_group_norm_kernel<bf16_t>, grid, dim3(256), 0, (hipStream_t)stream, x, ldx, gain, (const bf16_t*)gate,
+                               ldg, (bf16_t*)out, ldo, eps, cols, group_cols, pairs);
+        else
+            hipLaunchKernelGGL(gated_group_norm_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, x, ldx, gain, (const float*)gate,
+                               ldg, (float*)out, ldo, eps, cols, group_cols, pairs);
+        return pcb_check_launch("gated_group_norm_kernel");
+    }
     if (dtype == PCB_BF16)
         hipLaunchKernelGGL(gated_norm_kernel<bf16_t>, dim3(n_rows), dim3(256), 0, (hipStream_t)stream, x, ldx, gain, (const bf16_t*)gate,
                            ldg, (bf16_t*)out, ldo, eps, cols);
@@ -559,4 +656,20 @@ PCB_EXPORT int pcb_moe_mix(const float* pair_out, const int32_t* expert, const f
         hipLaunchKernelGGL(moe_mix_kernel<float>, dim3(n_rows), dim3(256), 0, (hipStream_t)stream, pair_out, expert, weight,
                            (const float*)h, n_real, y, width, top);
     return pcb_check_launch("moe_mix_kernel");
+}
+
+PCB_EXPORT int pcb_post_norm(const pcb_post_norm_args* a, void* stream) {
+    PCB_REQUIRE(a && a->struct_bytes == sizeof(pcb_post_norm_args), PCB_ERR_ARG, "pcb_post_norm: struct size mismatch");
+    PCB_REQUIRE(PCB_DTYPE_OK(a->dtype) && a->n_rows >= 0 && a->width > 0 && a->width <= 16384, PCB_ERR_ARG,
+                "pcb_post_norm: bad sizes (width <= 16384)");
+    if (a->n_rows == 0) return PCB_OK;
+    PCB_REQUIRE(a->x && (!a->out || a->gain) && (!a->gate || (a->y && a->ldg >= a->width)) && (!a->post_gain || a->y), PCB_ERR_ARG,
+                "pcb_post_norm: null pointer (a gate and a norm after the sublayer need its result, a norm its gain)");
+    const size_t lds = (size_t)a->width * sizeof(float);
+    const dim3 threads(a->n_rows <= 512 && a->width > 1024 ? 1024 : 256);
+    if (a->dtype == PCB_BF16)
+        hipLaunchKernelGGL(post_norm_kernel<bf16_t>, dim3(a->n_rows), threads, lds, (hipStream_t)stream, *a);
+    else
+        hipLaunchKernelGGL(post_norm_kernel<float>, dim3(a->n_rows), threads, lds, (hipStream_t)stream, *a);
+    return pcb_check_launch("post_norm_kernel");
 }

@@ -16,10 +16,10 @@ _lib: Optional[C.CDLL] = None
 
 BF16, F32 = 0, 1
 EPI_STORE, EPI_SILU_MUL, EPI_SCALE_ADD = 0, 1, 2
-ACT_NONE, ACT_SILU, ACT_SIGMOID, ACT_RELU2, ACT_SOFTPLUS, ACT_SOFTCAP = 0, 1, 2, 3, 4, 5
+ACT_NONE, ACT_SILU, ACT_SIGMOID, ACT_RELU2, ACT_SOFTPLUS, ACT_SOFTCAP, ACT_RELU, ACT_GELU_TANH = 0, 1, 2, 3, 4, 5, 6, 7
 NORM_NONE, NORM_RMS, NORM_DYT = 0, 1, 2
 SCORE_SIGMOID, SCORE_SOFTMAX = 0, 1
-ABI_VERSION = 2
+ABI_VERSION = 3
 DTYPES = {torch.bfloat16: BF16, torch.float32: F32}
 
 
@@ -42,7 +42,7 @@ class LinearArgs(C.Structure):
                 ("base", _vp), ("ldbase", _i64), ("col_scale", _vp),
                 ("split_n", _i32), ("y2", _vp), ("row_off2", _vp), ("head_dim2", _i32), ("head_stride2", _i64),
                 ("split_n3", _i32), ("y3", _vp), ("row_off3", _vp), ("col_stride3", _i64),
-                ("act", _i32), ("act_split", _i32), ("act2", _i32), ("act_param", _f32)]
+                ("act", _i32), ("act_split", _i32), ("act2", _i32), ("act_param", _f32), ("bias2", _vp)]
 
 
 class AttnTalkArgs(C.Structure):
@@ -72,7 +72,8 @@ class AttnSoftmaxArgs(C.Structure):
                 ("kcache", _vp), ("vcache", _vp), ("slot_stride", _i64), ("head_stride", _i64), ("row_stride", _i64),
                 ("v_slot_stride", _i64), ("v_head_stride", _i64), ("v_stride", _i64), ("v_cols", _i32),
                 ("H", _i32), ("Hkv", _i32), ("dim", _i32), ("vdim", _i32), ("scale", _f32), ("window", _i32),
-                ("gate", _vp), ("ldg", _i64), ("out", _vp), ("ldo", _i64), ("n_splits", _i32), ("part", _vp)]
+                ("gate", _vp), ("ldg", _i64), ("out", _vp), ("ldo", _i64), ("n_splits", _i32), ("part", _vp),
+                ("block", _i32), ("sink", _vp), ("gate_per_head", _i32)]
 
 
 class DecayAttnArgs(C.Structure):
@@ -91,11 +92,42 @@ class SelectiveScanArgs(C.Structure):
                 ("state", _vp), ("slot_stride", _i64), ("C", _i32), ("N", _i32), ("out", _vp), ("ldo", _i64), ("dt_sum", _vp)]
 
 
+class PostNormArgs(C.Structure):
+    """``pcb_post_norm_args`` (field for field)."""
+    _fields_ = [("struct_bytes", C.c_uint32), ("dtype", _i32),
+                ("x", _vp), ("y", _vp), ("gate", _vp), ("ldg", _i64), ("post_gain", _vp), ("gain", _vp),
+                ("out", _vp), ("x_out", _vp), ("rows", _vp), ("eps", _f32), ("n_rows", _i32), ("width", _i32)]
+
+
+class HeadPrepSeg(C.Structure):
+    """``pcb_head_prep_seg`` (field for field)."""
+    _fields_ = [("src", _vp), ("ld_src", _i64), ("src_head_stride", _i64), ("heads", _i32), ("head_dim", _i32), ("norm", _i32), ("gain", _vp),
+                ("blend", _vp), ("other", _vp), ("ld_other", _i64), ("keep", _vp), ("ld_keep", _i64),
+                ("rot_off", _i32), ("rot_dims", _i32), ("dst", _vp), ("ld_dst", _i64), ("row_off", _vp),
+                ("head_stride", _i64), ("col_stride", _i64)]
+
+
+class HeadPrepArgs(C.Structure):
+    """``pcb_head_prep_args`` (field for field)."""
+    _fields_ = [("struct_bytes", C.c_uint32), ("dtype", _i32), ("n_rows", _i32), ("n_segs", _i32),
+                ("pos", _vp), ("freqs", _vp), ("rot_mag", _f32), ("eps", _f32), ("seg", HeadPrepSeg * 4)]
+
+
+class MlstmArgs(C.Structure):
+    """``pcb_mlstm_args`` (field for field)."""
+    _fields_ = [("struct_bytes", C.c_uint32), ("dtype", _i32),
+                ("q", _vp), ("k", _vp), ("v", _vp), ("gi", _vp), ("gf", _vp),
+                ("ldq", _i64), ("ldk", _i64), ("ldv", _i64), ("ldgi", _i64), ("ldgf", _i64),
+                ("reqs", _vp), ("n_reqs", _i32), ("state", _vp), ("slot_stride", _i64),
+                ("H", _i32), ("dim", _i32), ("vdim", _i32), ("q_scale", _f32), ("gate_cap", _f32), ("out", _vp), ("ldo", _i64)]
+
+
 # name -> (restype, argtypes); mirrors include/promptcache_blocks.h one to one
 SIGNATURES = {
     "pcb_version": (C.c_int, []),
     "pcb_last_error_string": (C.c_char_p, []),
     "pcb_embed_rows": (C.c_int, [_vp, _i32, _vp, _vp, _i32, _i32, _i32, _vp]),
+    "pcb_embed_scaled_rows": (C.c_int, [_vp, _i32, _vp, _f32, _vp, _i32, _i32, _i32, _vp]),
     "pcb_mix_norm": (C.c_int, [C.POINTER(MixNormArgs), _vp]),
     "pcb_linear": (C.c_int, [C.POINTER(LinearArgs), _vp]),
     "pcb_polynorm": (C.c_int, [_vp, _vp, _vp, _i32, _f32, _i32, _i32, _vp]),
@@ -106,7 +138,7 @@ SIGNATURES = {
     "pcb_attn_talk": (C.c_int, [C.POINTER(AttnTalkArgs), _vp]),
     "pcb_embed_pos_rows": (C.c_int, [_vp, _vp, _i32, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _i32, _vp]),
     "pcb_hyper_norm": (C.c_int, [C.POINTER(HyperNormArgs), _vp]),
-    "pcb_gated_norm": (C.c_int, [_vp, _i64, _vp, _vp, _i64, _vp, _i64, _i32, _f32, _i32, _i32, _vp]),
+    "pcb_gated_norm": (C.c_int, [_vp, _i64, _vp, _vp, _i64, _vp, _i64, _i32, _f32, _i32, _i32, _i32, _vp]),
     "pcb_router_select": (C.c_int, [_vp, _i32, _i32, _i32, _i32, _vp, _i32, _i32, _i32, _vp, _vp, _vp]),
     "pcb_moe_mix": (C.c_int, [_vp, _vp, _vp, _vp, _i32, _i32, _vp, _i32, _i32, _i32, _vp]),
     "pcb_attn_softmax": (C.c_int, [C.POINTER(AttnSoftmaxArgs), _vp]),
@@ -115,6 +147,9 @@ SIGNATURES = {
     "pcb_conv_state_update": (C.c_int, [_vp, _i64, _i32, _vp, _i32, _vp, _i64, _i32, _i32, _vp]),
     "pcb_selective_scan": (C.c_int, [C.POINTER(SelectiveScanArgs), _vp]),
     "pcb_state_chain": (C.c_int, [_vp, _vp, _vp, _i64, _vp, _i32, _vp, _vp, _i32, _i32, _vp]),
+    "pcb_post_norm": (C.c_int, [C.POINTER(PostNormArgs), _vp]),
+    "pcb_head_prep": (C.c_int, [C.POINTER(HeadPrepArgs), _vp]),
+    "pcb_mlstm": (C.c_int, [C.POINTER(MlstmArgs), _vp]),
 }
 
 
@@ -176,6 +211,15 @@ def embed_rows(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> Non
     check(load().pcb_embed_rows(_p(table), _code(table), _p(ids), _p(out), n, width, table.shape[0], _stream()), "pcb_embed_rows")
 
 
+def embed_scaled_rows(table: torch.Tensor, ids: torch.Tensor, scale: float, out: torch.Tensor) -> None:
+    """``out`` fp32 [rows, width] = scale * table[ids]."""
+    n, width = out.shape
+    _want(ids, torch.int32, "embed_scaled_rows ids"); _want(out, torch.float32, "embed_scaled_rows out")
+    assert ids.numel() >= n and table.shape[1] == width and table.is_contiguous()
+    check(load().pcb_embed_scaled_rows(_p(table), _code(table), _p(ids), float(scale), _p(out), n, width, table.shape[0], _stream()),
+          "pcb_embed_scaled_rows")
+
+
 def mix_norm(hist: torch.Tensor, n_streams: int, coef: Optional[torch.Tensor], gain1: Optional[torch.Tensor],
              out1: Optional[torch.Tensor], gain2: Optional[torch.Tensor] = None, out2: Optional[torch.Tensor] = None,
              x_out: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None, eps: float = 1e-6,
@@ -205,14 +249,15 @@ def linear(x: torch.Tensor, w: torch.Tensor, y: torch.Tensor, *, M: int, epilogu
            row_src=None, row_scale=None, group_off=None, n_groups: int = 0, row_dst=None, base=None, col_scale=None,
            split_n: int = 0, y2=None, row_off2=None, head_dim2: int = 0, head_stride2: int = 0, split_n3: int = 0, y3=None,
            row_off3=None, col_stride3: int = 0, act: int = ACT_NONE,
-           act_split: int = 0, act2: int = ACT_NONE, act_param: float = 0.0, ldy: Optional[int] = None) -> None:
+           act_split: int = 0, act2: int = ACT_NONE, act_param: float = 0.0, ldy: Optional[int] = None, bias2=None,
+           ldx: Optional[int] = None) -> None:
     """``w``: [N, K], or [groups, N, K] with ``group_off``.  ``x``: [rows, K] of the weights' element type.  ``act`` (and ``act2``
     from column ``act_split`` on): the element-wise function of a plain store.  ``ldy``: row stride of ``y`` when it is a
     column block of a wider matrix."""
     code = _code(w)
-    assert x.dtype == w.dtype and x.is_contiguous() and w.is_contiguous() and x.is_cuda and w.is_cuda
+    assert x.dtype == w.dtype and (x.is_contiguous() or ldx is not None) and w.is_contiguous() and x.is_cuda and w.is_cuda
     N, K = w.shape[-2], w.shape[-1]
-    assert x.shape[-1] == K
+    assert x.shape[-1] == K or (ldx is not None and ldx >= K)
     if n_groups:
         assert w.dim() == 3 and w.shape[0] == n_groups and group_off is not None and group_off.numel() == n_groups + 1
         _want(group_off, torch.int32, "linear group_off")
@@ -220,8 +265,9 @@ def linear(x: torch.Tensor, w: torch.Tensor, y: torch.Tensor, *, M: int, epilogu
         assert w.dim() == 2
     if w2 is not None:
         assert w2.shape == w.shape and w2.dtype == w.dtype and w2.is_contiguous()
-    if bias is not None:
-        assert bias.dtype == w.dtype and bias.numel() == N
+    for b_ in (bias, bias2):
+        if b_ is not None:
+            assert b_.dtype == w.dtype and b_.numel() == N and b_.is_cuda
     for t, nm in ((row_src, "row_src"), (row_dst, "row_dst")):
         if t is not None:
             _want(t, torch.int32, "linear " + nm)
@@ -248,10 +294,10 @@ def linear(x: torch.Tensor, w: torch.Tensor, y: torch.Tensor, *, M: int, epilogu
     if split_n3:
         _want(row_off3, torch.int64, "linear row_off3")
         assert y3 is not None and y3.dtype == w.dtype and row_off3.numel() >= M and col_stride3 > 0 and split_n3 > split_n
-    a = LinearArgs(C.sizeof(LinearArgs), code, epilogue, _p(x), K, _p(row_src), _p(row_scale), _p(w), _p(w2), K, _p(bias),
+    a = LinearArgs(C.sizeof(LinearArgs), code, epilogue, _p(x), K if ldx is None else ldx, _p(row_src), _p(row_scale), _p(w), _p(w2), K, _p(bias),
                    M, N, K, _p(group_off), n_groups, N * K if n_groups else 0, _p(y), y.shape[-1] if ldy is None else ldy, out_f32,
                    _p(row_dst), _p(base), N, _p(col_scale), split_n, _p(y2), _p(row_off2), head_dim2, head_stride2,
-                   split_n3, _p(y3), _p(row_off3), col_stride3, int(act), int(act_split), int(act2), float(act_param))
+                   split_n3, _p(y3), _p(row_off3), col_stride3, int(act), int(act_split), int(act2), float(act_param), _p(bias2))
     check(load().pcb_linear(C.byref(a), _stream()), "pcb_linear")
 
 
@@ -355,16 +401,18 @@ def hyper_norm(streams: torch.Tensor, *, y=None, mix=None, out_w=None, in_w=None
 
 
 def gated_norm(x: torch.Tensor, gain: Optional[torch.Tensor], gate: Optional[torch.Tensor], ldg: int, out: torch.Tensor, eps: float,
-               n_rows: int) -> None:
-    """``x`` fp32 [rows, cols]; ``gate`` E, a column block (row stride ``ldg``) of a wider matrix; ``out`` E [rows, cols]."""
+               n_rows: int, group: int = 0) -> None:
+    """``x`` fp32 [rows, cols]; ``gate`` E, a column block (row stride ``ldg``) of a wider matrix; ``out`` E [rows, cols].
+    ``group`` > 0: a norm per run of that many columns (per head) instead of one over the row."""
     _want(x, torch.float32, "gated_norm x"); _want(gain, torch.float32, "gated_norm gain")
     cols = x.shape[-1]
     assert out.is_contiguous() and out.shape[-1] == cols and x.shape[0] >= n_rows and out.shape[0] >= n_rows
     assert gain is None or gain.numel() == cols
     if gate is not None:
         assert gate.dtype == out.dtype and gate.is_cuda and ldg >= cols
-    check(load().pcb_gated_norm(_p(x), cols, _p(gain), _p(gate), ldg, _p(out), cols, _code(out), float(eps), n_rows, cols, _stream()),
-          "pcb_gated_norm")
+    assert group == 0 or cols % group == 0
+    check(load().pcb_gated_norm(_p(x), cols, _p(gain), _p(gate), ldg, _p(out), cols, _code(out), float(eps), n_rows, cols, int(group),
+                                _stream()), "pcb_gated_norm")
 
 
 def router_select(logits: torch.Tensor, top: int, expert: torch.Tensor, weight: torch.Tensor, n_rows: int, *, score_fn: int,
@@ -391,22 +439,26 @@ def moe_mix(pair_out: torch.Tensor, expert: torch.Tensor, weight: torch.Tensor, 
 def attn_softmax(q: torch.Tensor, ldq: int, tiles: torch.Tensor, n_tiles: int, kcache: torch.Tensor, k_strides, vcache: torch.Tensor,
                  v_offset: int, v_strides, v_cols: bool, H: int, Hkv: int, dim: int, vdim: int, scale: float, out: torch.Tensor, *,
                  q_scale: Optional[torch.Tensor] = None, window: int = 0, gate: Optional[torch.Tensor] = None, ldg: int = 0,
-                 n_splits: int = 1, part: Optional[torch.Tensor] = None) -> None:
+                 n_splits: int = 1, part: Optional[torch.Tensor] = None, block: int = 0, sink: Optional[torch.Tensor] = None,
+                 gate_per_head: bool = False) -> None:
     """``q``: E rows (row stride ``ldq``, head h at column h * dim); ``kcache`` with ``k_strides`` = (slot, head, row) strides in
     elements; the values start ``v_offset`` elements into ``vcache`` (which may be the same plane) with ``v_strides`` = (slot, head,
     row) strides, or (slot, head, column) strides when ``v_cols`` (a cache kept column by column, columns readable in multiples of
     32 keys); ``gate``: E rows of stride ``ldg``; ``out`` E [rows, H * vdim].  ``n_splits`` > 1: each (tile, head) runs as that many
     workgroups over runs of the keys, merged by a second launch; ``part``: fp32 scratch of ``attn_softmax_part(rows, H, n_splits,
-    vdim)`` floats."""
+    vdim)`` floats.  ``block`` > 0: a key is seen only inside the query's own block of that many positions; ``sink`` fp32 [H]: one
+    more exp(sink[h]) in the denominator; ``gate_per_head``: the gate has one column per head."""
     _want(tiles, torch.int32, "attn_softmax tiles"); _want(q_scale, torch.float32, "attn_softmax q_scale")
+    _want(sink, torch.float32, "attn_softmax sink")
+    assert sink is None or sink.numel() == H
     assert q.dtype == kcache.dtype == vcache.dtype == out.dtype and out.is_contiguous() and kcache.is_cuda and vcache.is_cuda and q.is_cuda
     assert tiles.numel() >= 4 * n_tiles and out.shape[-1] == H * vdim and ldq >= H * dim
-    assert gate is None or (gate.dtype == q.dtype and ldg >= H * vdim)
+    assert gate is None or (gate.dtype == q.dtype and ldg >= (H if gate_per_head else H * vdim))
     es = vcache.element_size()
     a = AttnSoftmaxArgs(C.sizeof(AttnSoftmaxArgs), _code(q), _p(q), ldq, _p(q_scale), _p(tiles), n_tiles, _p(kcache),
                         vcache.data_ptr() + v_offset * es, int(k_strides[0]), int(k_strides[1]), int(k_strides[2]), int(v_strides[0]),
                         int(v_strides[1]), int(v_strides[2]), int(v_cols), H, Hkv, dim, vdim, float(scale), int(window), _p(gate), ldg,
-                        _p(out), out.shape[-1], int(n_splits), _p(part))
+                        _p(out), out.shape[-1], int(n_splits), _p(part), int(block), _p(sink), int(gate_per_head))
     if n_splits > 1:
         _want(part, torch.float32, "attn_softmax part")
         assert part.numel() >= attn_softmax_part(out.shape[0], H, n_splits, vdim)
@@ -483,3 +535,84 @@ def state_chain(local: torch.Tensor, start: torch.Tensor, state: torch.Tensor, c
     assert elems % group == 0 and x.numel() >= n_seg * (elems // group)
     check(load().pcb_state_chain(_p(local), _p(start), _p(state), elems, _p(chains), n_chains, _p(coef), _p(x), elems, group, _stream()),
           "pcb_state_chain")
+
+
+# ---- sublayers between two norms, per-head preparation, matrix memories ----------------------------------------------------------
+def post_norm(x: torch.Tensor, *, y=None, gate=None, ldg: int = 0, post_gain=None, gain=None, out=None, x_out=None, rows=None,
+              eps: float = 1e-6, n_rows: Optional[int] = None) -> None:
+    """``x`` fp32 [T, W] (the residual).  With ``y`` (fp32 [T, W]): x += norm(y * gate) * post_gain (``gate`` E rows of stride
+    ``ldg``; without ``post_gain`` the gated y is added as it is).  With ``out`` (E): out = norm(x) * gain, for the rows ``rows``
+    only if given (then x itself is not rewritten); ``x_out`` fp32 receives those rows of x."""
+    _want(x, torch.float32, "post_norm x")
+    T, W = x.shape
+    n = (rows.numel() if rows is not None else T) if n_rows is None else n_rows
+    for t, nm in ((y, "y"), (post_gain, "post_gain"), (gain, "gain"), (x_out, "x_out")):
+        _want(t, torch.float32, "post_norm " + nm)
+    assert rows is not None or n <= T
+    if y is not None:
+        assert y.shape[-1] == W and y.shape[0] >= (T if rows is not None else n)
+    if gate is not None:
+        assert y is not None and gate.is_cuda and ldg >= W and gate.dtype in DTYPES
+    code = _code(out) if out is not None else (_code(gate) if gate is not None else BF16)
+    if out is not None:
+        assert out.is_contiguous() and out.shape[-1] == W and out.numel() >= n * W and gain is not None and gain.numel() == W
+        assert gate is None or gate.dtype == out.dtype
+    assert post_gain is None or post_gain.numel() == W
+    if x_out is not None:
+        assert x_out.numel() >= n * W
+    if rows is not None:
+        _want(rows, torch.int32, "post_norm rows")
+    a = PostNormArgs(C.sizeof(PostNormArgs), code, _p(x), _p(y), _p(gate), ldg, _p(post_gain), _p(gain), _p(out), _p(x_out), _p(rows),
+                     float(eps), n, W)
+    check(load().pcb_post_norm(C.byref(a), _stream()), "pcb_post_norm")
+
+
+def head_seg(src: torch.Tensor, ld_src: int, heads: int, head_dim: int, dst: torch.Tensor, *, norm: bool = False, gain=None, blend=None,
+             other=None, keep=None, rot_off: int = 0, rot_dims: int = 0, ld_dst: int = 0, row_off=None, head_stride: Optional[int] = None,
+             col_stride: int = 1, dst_offset: int = 0, src_head_stride: Optional[int] = None) -> HeadPrepSeg:
+    """One segment of ``head_prep``: ``src`` E, a column block (row stride ``ld_src``) whose first ``heads * head_dim`` columns are
+    the heads; ``dst`` E: a row matrix (``ld_dst``, heads ``head_stride`` apart, starting ``dst_offset`` elements in) or a cache
+    (``row_off`` int64 per row; ``col_stride`` > 1 for one kept column by column).  ``other`` / ``keep``: fp32 [rows, heads *
+    head_dim]."""
+    for t, nm in ((gain, "gain"), (blend, "blend"), (other, "other"), (keep, "keep")):
+        _want(t, torch.float32, "head_prep " + nm)
+    _want(row_off, torch.int64, "head_prep row_off")
+    shs = head_dim if src_head_stride is None else src_head_stride
+    assert src.dtype == dst.dtype and src.is_cuda and dst.is_cuda and ld_src >= (heads - 1) * shs + head_dim
+    assert gain is None or gain.numel() == head_dim
+    assert blend is None or (other is not None and other.shape[-1] == heads * head_dim)
+    assert keep is None or keep.shape[-1] == heads * head_dim
+    assert row_off is not None or ld_dst > 0
+    return HeadPrepSeg(_p(src), ld_src, shs, heads, head_dim, int(norm), _p(gain), _p(blend), _p(other), heads * head_dim, _p(keep),
+                       heads * head_dim, rot_off, rot_dims, dst.data_ptr() + dst_offset * dst.element_size(), ld_dst, _p(row_off),
+                       head_dim if head_stride is None else head_stride, col_stride)
+
+
+def head_prep(segs, n_rows: int, dtype, *, pos: Optional[torch.Tensor] = None, freqs: Optional[torch.Tensor] = None, rot_mag: float = 1.0,
+              eps: float = 1e-6) -> None:
+    """``segs``: one to four ``head_seg`` records; ``pos`` int32 [rows]; ``freqs`` float64 [rot_dims / 2]."""
+    _want(pos, torch.int32, "head_prep pos"); _want(freqs, torch.float64, "head_prep freqs")
+    assert 1 <= len(segs) <= 4
+    rot = {s.rot_dims for s in segs if s.rot_dims}
+    assert len(rot) <= 1 and (not rot or (pos is not None and freqs is not None and pos.numel() >= n_rows and 2 * freqs.numel() == rot.pop()))
+    a = HeadPrepArgs(C.sizeof(HeadPrepArgs), DTYPES[dtype], n_rows, len(segs), _p(pos), _p(freqs), float(rot_mag), float(eps))
+    for i, sg in enumerate(segs):
+        a.seg[i] = sg
+    check(load().pcb_head_prep(C.byref(a), _stream()), "pcb_head_prep")
+
+
+def mlstm_state_floats(H: int, dim: int, vdim: int) -> int:
+    """fp32 elements of a slot's state: per head S [dim][vdim], then n [dim], then the running maximum."""
+    return H * (dim * vdim + dim + 1)
+
+
+def mlstm(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gi: torch.Tensor, gf: torch.Tensor, ld: int, reqs: torch.Tensor, n_reqs: int,
+          state: torch.Tensor, H: int, dim: int, vdim: int, q_scale: float, gate_cap: float, out: Optional[torch.Tensor]) -> None:
+    """``q``, ``k``, ``v``, ``gi``, ``gf``: column blocks (row stride ``ld``) of one E matrix; ``state`` fp32 [slots,
+    mlstm_state_floats]; ``out`` fp32 [rows, H * vdim]."""
+    _want(reqs, torch.int32, "mlstm reqs"); _want(state, torch.float32, "mlstm state"); _want(out, torch.float32, "mlstm out")
+    assert q.dtype == k.dtype == v.dtype == gi.dtype == gf.dtype and q.is_cuda and reqs.numel() >= 4 * n_reqs
+    assert state[0].numel() == mlstm_state_floats(H, dim, vdim) and (out is None or out.shape[-1] == H * vdim)
+    a = MlstmArgs(C.sizeof(MlstmArgs), _code(q), _p(q), _p(k), _p(v), _p(gi), _p(gf), ld, ld, ld, ld, ld, _p(reqs), n_reqs, _p(state),
+                  state[0].numel(), H, dim, vdim, float(q_scale), float(gate_cap), _p(out), H * vdim)
+    check(load().pcb_mlstm(C.byref(a), _stream()), "pcb_mlstm")

@@ -389,42 +389,3 @@ class DibizenHIP(SlotModel):
             B.linear(h, lw["up"], act, M=P, row_src=row_src, group_off=goff[:l.experts + 1], n_groups=l.experts, act=B.ACT_RELU2)
             B.linear(act, lw["down"], pair, M=P, row_dst=row_dst, group_off=goff[:l.experts + 1], n_groups=l.experts)
         B.moe_mix(pair, expert, weight, h, l.experts, y, T, l.top)
-
-    # ---- decode steps as captured graphs -----------------------------------------------------------------------------------------
-    def _decode_graphed(self, arena, blob, d):
-        """A step of T requests with one token each, replayed from a hipGraph captured per (T, arena planes).  What changes
-        between steps -- tokens, slots, positions -- lives in the step's tables, which the graph reads from a device block that
-        one copy from pinned memory refreshes; no launch dimension depends on the requests' lengths."""
-        T = d["T"]
-        key = (T, id(arena), arena.generation)
-        ent = self._graphs.pop(key, None)
-        if ent is None:
-            for k in [k for k in self._graphs if k[1] == id(arena) and k[2] != arena.generation]:
-                del self._graphs[k]                               # graphs over planes that have moved
-            while len(self._graphs) >= self.max_graphs:
-                self._graphs.pop(next(iter(self._graphs)))
-            ent = dict(graph=None, bufs={}, host=torch.empty(blob.size, dtype=torch.uint8, pin_memory=True),
-                       dev=torch.empty(blob.size, dtype=torch.uint8, device=self.device),
-                       logits=torch.empty((T, self.V), dtype=torch.float32, device=self.device), copied=torch.cuda.Event())
-        self._graphs[key] = ent                                   # (re-inserted at the young end)
-        ent["copied"].synchronize()                               # the previous step's upload has left the pinned block
-        ent["host"].numpy()[:] = blob
-        ent["dev"].copy_(ent["host"], non_blocking=True)
-        ent["copied"].record()
-        if ent["graph"] is None:
-            from .llama_hip import prime_graph_capture
-            saved, self._buf = self._buf, ent["bufs"]             # the graph owns its scratch
-            try:
-                self._run(arena, ent["dev"], d, ent["logits"])    # eager first: sizes every scratch buffer, and is this step's result
-                torch.cuda.synchronize()
-                # (capture records the launches without executing them: the recurrent states advance once, by the eager run)
-                prime_graph_capture(self.device)
-                g = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(g):
-                    self._run(arena, ent["dev"], d, ent["logits"])
-                ent["graph"] = g
-            finally:
-                self._buf = saved
-            return ent["logits"].clone()
-        ent["graph"].replay()
-        return ent["logits"].clone()

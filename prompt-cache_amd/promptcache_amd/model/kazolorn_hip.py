@@ -255,10 +255,10 @@ class KazolornHIP(SlotModel):
         worst = max(16 * T * l.heads * B.attn_talk_band(l.window, cap) for l in self.config.layers)
         if worst > ATTN_SCRATCH_FLOATS // 4:
             return None
-        key = (T, id(arena), arena.generation)
+        key = (T, arena.serial, arena.generation)
         ent = self._graphs.pop(key, None)
         if ent is None:
-            for k in [k for k in self._graphs if k[1] == id(arena) and k[2] != arena.generation]:
+            for k in [k for k in self._graphs if k[1] == arena.serial and k[2] != arena.generation]:
                 del self._graphs[k]                               # graphs over planes that have moved
             while len(self._graphs) >= self.max_graphs:
                 self._graphs.pop(next(iter(self._graphs)))

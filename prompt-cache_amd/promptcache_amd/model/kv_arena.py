@@ -293,7 +293,13 @@ class SlotArena:
     ``self.states[layer]``.  A state is not cleared when its slot changes hands: whoever reads it treats a request that starts
     at position 0 as starting from zero."""
 
+    _serials = 0
+
     def __init__(self, layer_dims, slots: int, cap: int, device, dtype=torch.bfloat16, states=None, col_dims=None):
+        # a number no other arena of this process has or had: what captured launches are filed under (an object's address can
+        # come back after the object is gone, with other planes behind it)
+        SlotArena._serials += 1
+        self.serial = SlotArena._serials
         self.layer_dims = [(int(g), int(d)) for g, d in layer_dims]
         # a second plane per layer kept COLUMN by column, ``[slots][heads][columns][cap]`` (values whose readers want a run of
         # positions of one column contiguous); with any of these, cap is kept a multiple of 32 so that a reader may fetch whole

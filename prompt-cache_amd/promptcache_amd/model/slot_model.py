@@ -31,7 +31,8 @@ class SlotKV:
 
 class SlotModel:
     """Mixin of the flat-row models.  The subclass provides ``device``, ``dtype``, ``V`` (vocabulary), ``decode_headroom``,
-    ``default_arena``, ``_buf`` (scratch by name), ``new_arena(slots, cap)`` and ``forward_rows``."""
+    ``default_arena``, ``_buf`` (scratch by name), ``new_arena(slots, cap)`` and ``forward_rows``; one that replays its one-token
+    steps from captured graphs (``_decode_graphed``) also ``_graphs``, ``max_graphs`` and ``_run``."""
 
     # ---- scratch -----------------------------------------------------------------------------------------------------------
     def _scratch(self, name: str, numel: int, dtype) -> torch.Tensor:
@@ -45,6 +46,45 @@ class SlotModel:
 
     def _mat(self, name: str, rows: int, cols: int, dtype) -> torch.Tensor:
         return self._scratch(name, max(rows, 1) * cols, dtype)[:max(rows, 1) * cols].view(max(rows, 1), cols)
+
+    # ---- one-token steps as captured graphs (models whose step is ``_run(arena, device tables, dims, logits)``) ------------------
+    def _decode_graphed(self, arena, blob, d):
+        """A step of T requests with one token each, replayed from a hipGraph captured per (T, arena planes).  What changes
+        between steps -- tokens, slots, positions -- lives in the step's tables, which the graph reads from a device block that
+        one copy from pinned memory refreshes; no launch dimension depends on the requests' lengths."""
+        T = d["T"]
+        key = (T, arena.serial, arena.generation)
+        ent = self._graphs.pop(key, None)
+        if ent is None:
+            for k in [k for k in self._graphs if k[1] == arena.serial and k[2] != arena.generation]:
+                del self._graphs[k]                               # graphs over planes that have moved
+            while len(self._graphs) >= self.max_graphs:
+                self._graphs.pop(next(iter(self._graphs)))
+            ent = dict(graph=None, bufs={}, host=torch.empty(blob.size, dtype=torch.uint8, pin_memory=True),
+                       dev=torch.empty(blob.size, dtype=torch.uint8, device=self.device),
+                       logits=torch.empty((T, self.V), dtype=torch.float32, device=self.device), copied=torch.cuda.Event())
+        self._graphs[key] = ent                                   # (re-inserted at the young end)
+        ent["copied"].synchronize()                               # the previous step's upload has left the pinned block
+        ent["host"].numpy()[:] = blob
+        ent["dev"].copy_(ent["host"], non_blocking=True)
+        ent["copied"].record()
+        if ent["graph"] is None:
+            from .llama_hip import prime_graph_capture
+            saved, self._buf = self._buf, ent["bufs"]             # the graph owns its scratch
+            try:
+                self._run(arena, ent["dev"], d, ent["logits"])    # eager first: sizes every scratch buffer, and is this step's result
+                torch.cuda.synchronize()
+                # (capture records the launches without executing them: the recurrent states advance once, by the eager run)
+                prime_graph_capture(self.device)
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    self._run(arena, ent["dev"], d, ent["logits"])
+                ent["graph"] = g
+            finally:
+                self._buf = saved
+            return ent["logits"].clone()
+        ent["graph"].replay()
+        return ent["logits"].clone()
 
     # ---- the adapters' calling convention --------------------------------------------------------------------------------------
     @torch.inference_mode()

@@ -438,3 +438,85 @@ def load_dibizen_safetensors(path: str, cfg):
         if tuple(raw[k].shape) != tuple(shp):
             raise ValueError(f"{path}: {k} has shape {tuple(raw[k].shape)}, the configuration implies {tuple(shp)}")
     return {k: raw[k] for k in want}
+
+
+def fivesun_weight_shapes(cfg) -> Dict[str, tuple]:
+    """Tensor names and shapes of a Fivesun checkpoint (``model.safetensors``): ``embed``; per layer ``l{i}.norm1|norm1b`` (the
+    norms before and after the mixer), ``l{i}.rg1`` (+ ``.b``: the sigmoid gate on the mixer's result), the mixer's ``l{i}.mix.*``
+    (attention: ``q k v q.norm k.norm sink g o`` and ``vmix`` when it blends values; latent_attention: ``q dkv dkv.norm uk uv g
+    o``; mlstm: ``q k v g o norm i i.b f f.b``) and, with a feed-forward, ``l{i}.norm2|norm2b``, ``l{i}.rg2`` (+ ``.b``) and
+    ``l{i}.mlp.gate|up|down`` (each with ``.b``); then ``final.norm`` and ``head``."""
+    W = cfg.hidden_size
+    s = {"embed": (cfg.vocab_size, W)}
+    for i, l in enumerate(cfg.layers):
+        p, m = f"l{i}.", f"l{i}.mix."
+        s[p + "norm1"], s[p + "norm1b"], s[p + "rg1"], s[p + "rg1.b"] = (W,), (W,), (W, W), (W,)
+        if l.kind == "attention":
+            s[m + "q"], s[m + "k"], s[m + "v"] = (l.heads * l.dim, W), (l.kv_heads * l.dim, W), (l.kv_heads * l.vdim, W)
+            s[m + "q.norm"], s[m + "k.norm"], s[m + "sink"] = (l.dim,), (l.dim,), (l.heads,)
+            s[m + "g"], s[m + "o"] = (l.heads, W), (W, l.heads * l.vdim)
+            if l.v_mix:
+                s[m + "vmix"] = ()
+        elif l.kind == "latent_attention":
+            s[m + "q"], s[m + "dkv"], s[m + "dkv.norm"] = (l.heads * (l.dim + l.rot_dim), W), (l.kv_rank + l.rot_dim, W), (l.kv_rank,)
+            s[m + "uk"], s[m + "uv"] = (l.heads * l.dim, l.kv_rank), (l.heads * l.vdim, l.kv_rank)
+            s[m + "g"], s[m + "o"] = (l.heads * l.vdim, W), (W, l.heads * l.vdim)
+        else:
+            s[m + "q"], s[m + "k"], s[m + "v"] = (l.heads * l.dim, W), (l.heads * l.dim, W), (l.heads * l.vdim, W)
+            s[m + "g"], s[m + "o"], s[m + "norm"] = (l.heads * l.vdim, W), (W, l.heads * l.vdim), (l.heads * l.vdim,)
+            s[m + "i"], s[m + "i.b"], s[m + "f"], s[m + "f.b"] = (l.heads, W), (l.heads,), (l.heads, W), (l.heads,)
+        if l.ff:
+            s[p + "norm2"], s[p + "norm2b"], s[p + "rg2"], s[p + "rg2.b"] = (W,), (W,), (W, W), (W,)
+            for nm, shp in (("gate", (l.ff, W)), ("up", (l.ff, W)), ("down", (W, l.ff))):
+                s[p + "mlp." + nm], s[p + "mlp." + nm + ".b"] = shp, (shp[0],)
+    s["final.norm"], s["head"] = (W,), (cfg.vocab_size, W)
+    return s
+
+
+def make_fivesun_weights(cfg, seed: int = 0, device="cpu", scale: float = 1.0):
+    """Seeded random weights (bfloat16 torch tensors) with nothing at a value that would hide a dropped term: norm gains around 1,
+    non-zero biases, sinks of both signs, blend weights strictly between 0 and 1, forget-gate biases that keep the memory for tens
+    of tokens."""
+    import torch
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    on_gpu = str(device) != "cpu"
+    gd = torch.Generator(device=device).manual_seed(seed) if on_gpu else g
+
+    def rnd(shape, big=False):
+        if big and on_gpu:
+            return torch.randn(shape, generator=gd, device=device, dtype=torch.float32)
+        return torch.randn(shape, generator=g, dtype=torch.float32).to(device)
+
+    out = {}
+    for name, shp in fivesun_weight_shapes(cfg).items():
+        leaf = name.split(".", 1)[-1] if name.startswith("l") and name[1].isdigit() else name
+        if leaf in ("norm1", "norm2", "norm1b", "norm2b", "final.norm", "mix.norm", "mix.q.norm", "mix.k.norm", "mix.dkv.norm"):
+            w = 1.0 + 0.1 * rnd(shp)
+        elif leaf == "mix.vmix":
+            w = torch.tensor(0.35, device=device) + 0.1 * rnd(shp)
+        elif leaf == "mix.sink":
+            w = 0.8 * rnd(shp)
+        elif leaf == "mix.f.b":
+            w = 3.0 + 0.5 * rnd(shp)
+        elif leaf.endswith(".b"):
+            w = 0.1 * rnd(shp)
+        elif leaf == "embed":
+            w = rnd(shp, big=True) / cfg.embed_scale
+        else:
+            w = (scale / (shp[-1] ** 0.5)) * rnd(shp, big=True)
+        out[name] = w.to(torch.bfloat16)
+    return out
+
+
+def load_fivesun_safetensors(path: str, cfg):
+    """The tensors of ``<path>/model.safetensors`` by their own names, on the host, checked against the shapes the
+    configuration implies."""
+    raw = read_checkpoint_dir(path)
+    want = fivesun_weight_shapes(cfg)
+    missing = [k for k in want if k not in raw]
+    if missing:
+        raise KeyError(f"{path}: tensors missing for this configuration: {missing[:6]}{' ...' if len(missing) > 6 else ''}")
+    for k, shp in want.items():
+        if tuple(raw[k].shape) != tuple(shp) and raw[k].numel() != 1:
+            raise ValueError(f"{path}: {k} has shape {tuple(raw[k].shape)}, the configuration implies {tuple(shp)}")
+    return {k: raw[k] for k in want}
