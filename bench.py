@@ -745,6 +745,45 @@ def run_dibizen(args):
     print(json.dumps(out))
 
 
+def run_fivesun(args):
+    """Throughput of the Fivesun stack beside the Dibizen stack (the closest existing model: the same building-block library, bf16
+    tensors, an fp32 residual, a gated softmax attention and a matrix-state recurrence among its mixers) at equal width, heads and
+    depth, with feed-forwards of equal work (Fivesun: a dense gated unit of 2 x width; Dibizen: 2 of 4 experts of 1.5 x width).
+
+    Per size: one prompt of 2048 tokens (tokens/s of the prefill), then decoding at a context of 2048 with 1 and 8 requests.
+    `mixed` = attention, latent attention, attention, mlstm; `attention` / `latent` / `mlstm` = four layers of that mixer alone,
+    which is what prices each mixer's kernels (beside Dibizen's `attention` and `lightning`).  Attention sees blocks of 1024
+    positions, latent attention a window of 1024 over a latent of 192 + 64 columns.  Random weights, synthetic tokens."""
+    import torch
+    import __graft_entry__ as ge
+    ge.build()
+    from promptcache_amd.model import Dibizen, Fivesun
+    from promptcache_amd.model.config import DibizenShape, FivesunShape
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    sizes = {"2k": dict(width=2048, heads=16, kv=4), "4k": dict(width=4096, heads=32, kv=8)}
+    L, V, T, steps, warm = 4, 32000, 2048, max(4, min(args.steps, 20)), max(1, min(args.warmup, 3))
+    g = torch.Generator().manual_seed(0)
+    out = {"metric": "fivesun_throughput", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "layers": L, "prompt": T, "sizes": {}}
+    patterns = {"mixed": ["attention", "latent_attention", "attention", "mlstm"], "attention": ["attention"] * L,
+                "latent": ["latent_attention"] * L, "mlstm": ["mlstm"] * L}
+    for key in args.fivesun_sizes.split(","):
+        c = sizes[key]
+        w, h = c["width"], c["heads"]
+        row = {"width": w, "heads": h}
+        for pk in (("attention", "lightning") if args.fivesun_baseline else ()):
+            dz = DibizenShape.uniform(V, w, [pk] * L, h, c["kv"], w // h, 4, 2, 3 * w // 2, streams=1, max_positions=T + 256,
+                                      name=f"dibizen-{key}-{pk}")
+            row["dibizen_" + pk] = slot_model_case(Dibizen(shape=dz, random_init=True, seed=0, device=dev), V, T, steps, warm, g)
+        for pk in args.fivesun_patterns.split(","):
+            shape = FivesunShape.uniform(V, w, patterns[pk], h, c["kv"], w // h, 2 * w, chunk=1024, window=1024, kv_rank=192, rot_dim=64,
+                                         name=f"fivesun-{key}-{pk}")
+            row["fivesun_" + pk] = slot_model_case(Fivesun(shape=shape, random_init=True, seed=0, device=dev), V, T, steps, warm, g)
+        out["sizes"][key] = row
+        print(json.dumps({key: row}), file=sys.stderr, flush=True)
+    print(json.dumps(out))
+
+
 def run_kazolorn(args):
     """Throughput of the Kazolorn stack beside the MPT stack at equal width, heads, depth and feed-forward width.
 
@@ -848,6 +887,12 @@ def main():
                          "real models (random weights), beside the Kazolorn stack (the closest existing model) at equal size")
     ap.add_argument("--dibizen-sizes", default="2k,4k", help="--dibizen: which sizes (2k, 4k)")
     ap.add_argument("--dibizen-patterns", default="mixed,attention,lightning,mamba1", help="--dibizen: which layer patterns")
+    ap.add_argument("--fivesun", action="store_true",
+                    help="instead of the default workload: prefill / decode throughput of the Fivesun design at layer sizes of "
+                         "real models (random weights), beside the Dibizen stack (the closest existing model) at equal size")
+    ap.add_argument("--fivesun-sizes", default="2k,4k", help="--fivesun: which sizes (2k, 4k)")
+    ap.add_argument("--fivesun-patterns", default="mixed,attention,latent,mlstm", help="--fivesun: which layer patterns")
+    ap.add_argument("--fivesun-baseline", type=int, default=1, help="--fivesun: 0 leaves the Dibizen stacks out (kernel profiles of Fivesun alone)")
     args = ap.parse_args()
     if args.plan_only:
         plan_only(args)
@@ -857,6 +902,9 @@ def main():
         return
     if args.dibizen:
         run_dibizen(args)
+        return
+    if args.fivesun:
+        run_fivesun(args)
         return
 
     import torch

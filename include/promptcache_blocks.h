@@ -439,7 +439,11 @@ int pcb_head_prep(const pcb_head_prep_args* a, void* stream);
  *   o = S'^T (q_scale q) / (max(|n' . q_scale q|, exp(-m')) + 1e-6)
  * q, k: E rows, head h at column h * dim; v: head h at column h * vdim; gi, gf: E rows, one column per head (the gates'
  * pre-activations, bias included); out fp32 [rows][ldo].  request r = {slot, first position, tokens, first flat row} as in
- * pcb_decay_attn.  state: fp32 per slot [H][dim * vdim + dim + 1] (S, then n, then m), slot_stride floats apart. */
+ * pcb_decay_attn.  state: fp32 per slot [H][dim * vdim + dim + 1] (S, then n, then m), slot_stride floats apart.
+ * out null: only the states move.  from_nothing: every request starts from S = n = 0 and m = -infinity whatever its position
+ * says (a segment's own contribution, see pcb_mlstm_chain); log_f_sum (fp32 [n_reqs][H], optional) receives each request's sum
+ * of log forget gates.  end_slots (int32 [n_reqs], optional): request r with end_slots[r] >= 0 leaves its last state in
+ * end_state + end_slots[r] * end_slot_stride instead of its own record (the last segment of a prompt writes the slot's state). */
 typedef struct pcb_mlstm_args {
     uint32_t struct_bytes;
     int32_t dtype;
@@ -458,8 +462,24 @@ typedef struct pcb_mlstm_args {
     float gate_cap;
     float* out;
     int64_t ldo;
+    int32_t from_nothing;
+    float* log_f_sum;
+    const int32_t* end_slots;
+    float* end_state;
+    int64_t end_slot_stride;
 } pcb_mlstm_args;
 int pcb_mlstm(const pcb_mlstm_args* a, void* stream);
+
+/* Segmented prefill of the matrix memory: a first pcb_mlstm pass runs every segment from nothing (local[g] = its contribution,
+ * log_f_sum[g] = its sum of log forget gates, both per head), this call chains them, and a second pass runs every segment from its
+ * true start state.  For chain c = {slot, first position, first segment, segments} (int32 x 4) and every head, with records
+ * (S, n, m) of dim * vdim + dim + 1 floats:
+ *   (S, n, m) = first position > 0 ? state[slot] : (0, 0, 0)
+ *   for g = first segment ..:  start[g] = (S, n, m);  m' = max(F_g + m, m_g);
+ *                              S <- exp(F_g + m - m') S + exp(m_g - m') S_g;  n likewise;  m <- m'
+ * local, start: fp32 [segments][H][record]; state is only read. */
+int pcb_mlstm_chain(const float* local, const float* log_f_sum, float* start, const float* state, int64_t slot_stride, const int32_t* chains,
+                    int32_t n_chains, int32_t H, int32_t dim, int32_t vdim, void* stream);
 
 #ifdef __cplusplus
 }

@@ -119,7 +119,8 @@ class MlstmArgs(C.Structure):
                 ("q", _vp), ("k", _vp), ("v", _vp), ("gi", _vp), ("gf", _vp),
                 ("ldq", _i64), ("ldk", _i64), ("ldv", _i64), ("ldgi", _i64), ("ldgf", _i64),
                 ("reqs", _vp), ("n_reqs", _i32), ("state", _vp), ("slot_stride", _i64),
-                ("H", _i32), ("dim", _i32), ("vdim", _i32), ("q_scale", _f32), ("gate_cap", _f32), ("out", _vp), ("ldo", _i64)]
+                ("H", _i32), ("dim", _i32), ("vdim", _i32), ("q_scale", _f32), ("gate_cap", _f32), ("out", _vp), ("ldo", _i64),
+                ("from_nothing", _i32), ("log_f_sum", _vp), ("end_slots", _vp), ("end_state", _vp), ("end_slot_stride", _i64)]
 
 
 # name -> (restype, argtypes); mirrors include/promptcache_blocks.h one to one
@@ -150,6 +151,7 @@ SIGNATURES = {
     "pcb_post_norm": (C.c_int, [C.POINTER(PostNormArgs), _vp]),
     "pcb_head_prep": (C.c_int, [C.POINTER(HeadPrepArgs), _vp]),
     "pcb_mlstm": (C.c_int, [C.POINTER(MlstmArgs), _vp]),
+    "pcb_mlstm_chain": (C.c_int, [_vp, _vp, _vp, _vp, _i64, _vp, _i32, _i32, _i32, _i32, _vp]),
 }
 
 
@@ -607,12 +609,35 @@ def mlstm_state_floats(H: int, dim: int, vdim: int) -> int:
 
 
 def mlstm(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gi: torch.Tensor, gf: torch.Tensor, ld: int, reqs: torch.Tensor, n_reqs: int,
-          state: torch.Tensor, H: int, dim: int, vdim: int, q_scale: float, gate_cap: float, out: Optional[torch.Tensor]) -> None:
+          state: torch.Tensor, H: int, dim: int, vdim: int, q_scale: float, gate_cap: float, out: Optional[torch.Tensor],
+          from_nothing: bool = False, log_f_sum: Optional[torch.Tensor] = None, end_slots: Optional[torch.Tensor] = None,
+          end_state: Optional[torch.Tensor] = None) -> None:
     """``q``, ``k``, ``v``, ``gi``, ``gf``: column blocks (row stride ``ld``) of one E matrix; ``state`` fp32 [slots,
-    mlstm_state_floats]; ``out`` fp32 [rows, H * vdim]."""
+    mlstm_state_floats]; ``out`` fp32 [rows, H * vdim], or None: only the states move.  ``from_nothing``: every request is a
+    segment that starts from an empty memory; ``log_f_sum`` fp32 [n_reqs, H] receives its sum of log forget gates.  ``end_slots``
+    int32 [n_reqs]: where >= 0, the request's last state goes to that slot of ``end_state`` instead of its own record."""
     _want(reqs, torch.int32, "mlstm reqs"); _want(state, torch.float32, "mlstm state"); _want(out, torch.float32, "mlstm out")
+    _want(log_f_sum, torch.float32, "mlstm log_f_sum")
+    assert log_f_sum is None or log_f_sum.numel() >= n_reqs * H
+    _want(end_slots, torch.int32, "mlstm end_slots"); _want(end_state, torch.float32, "mlstm end_state")
+    assert end_slots is None or (end_slots.numel() >= n_reqs and end_state is not None and end_state[0].numel() == state[0].numel())
     assert q.dtype == k.dtype == v.dtype == gi.dtype == gf.dtype and q.is_cuda and reqs.numel() >= 4 * n_reqs
     assert state[0].numel() == mlstm_state_floats(H, dim, vdim) and (out is None or out.shape[-1] == H * vdim)
     a = MlstmArgs(C.sizeof(MlstmArgs), _code(q), _p(q), _p(k), _p(v), _p(gi), _p(gf), ld, ld, ld, ld, ld, _p(reqs), n_reqs, _p(state),
-                  state[0].numel(), H, dim, vdim, float(q_scale), float(gate_cap), _p(out), H * vdim)
+                  state[0].numel(), H, dim, vdim, float(q_scale), float(gate_cap), _p(out), H * vdim, int(from_nothing), _p(log_f_sum),
+                  _p(end_slots), _p(end_state), end_state[0].numel() if end_state is not None else 0)
     check(load().pcb_mlstm(C.byref(a), _stream()), "pcb_mlstm")
+
+
+def mlstm_chain(local: torch.Tensor, log_f_sum: torch.Tensor, start: torch.Tensor, state: torch.Tensor, chains: torch.Tensor, n_chains: int,
+                H: int, dim: int, vdim: int) -> None:
+    """``local``, ``start`` fp32 [segments, mlstm_state_floats]; ``log_f_sum`` fp32 [segments, H]; ``state`` fp32 [slots,
+    mlstm_state_floats]; ``chains`` int32 {slot, first position, first segment, segments} x n_chains."""
+    for t, nm in ((local, "local"), (log_f_sum, "log_f_sum"), (start, "start"), (state, "state")):
+        _want(t, torch.float32, "mlstm_chain " + nm)
+    _want(chains, torch.int32, "mlstm_chain chains")
+    rec = mlstm_state_floats(H, dim, vdim)
+    assert local.shape[-1] == rec == start.shape[-1] == state[0].numel() and local.shape[0] == start.shape[0]
+    assert log_f_sum.numel() >= local.shape[0] * H and chains.numel() >= 4 * n_chains
+    check(load().pcb_mlstm_chain(_p(local), _p(log_f_sum), _p(start), _p(state), rec, _p(chains), n_chains, H, dim, vdim, _stream()),
+          "pcb_mlstm_chain")

@@ -563,7 +563,9 @@ class FivesunShape:
             if mlp:
                 if mlp.get("kind", "dense") != "dense":
                     raise ValueError(f"layer {i}: unknown feed-forward kind {mlp.get('kind')!r}")
-                lay.ff = int(mlp["ff"])
+                lay.ff, lay.act = int(mlp["ff"]), str(mlp.get("act", "relu"))
+                if lay.act not in ("relu", "silu", "gelu_tanh"):
+                    raise ValueError(f"layer {i}: unknown activation {lay.act!r}")
             layers.append(lay)
         shape = cls(vocab_size=int(c["vocab"]), hidden_size=int(c["width"]), norm_eps=float((c.get("norm") or {}).get("eps", 1e-6)),
                     layers=layers, embed_scale=float((c.get("embedding") or {}).get("scale", 1.0)), name=name)
@@ -601,7 +603,10 @@ class FivesunShape:
                 mixer = {"dim": l.dim, "gate_cap": l.gate_cap, "heads": l.heads, "vdim": l.vdim}
             if l.mask:
                 mixer["mask"] = {"size": l.mask}
-            out.append({"type": l.kind, "mixer": mixer, "mlp": {"ff": l.ff, "kind": "dense"} if l.ff else None})
+            mlp = {"ff": l.ff, "kind": "dense"} if l.ff else None
+            if mlp and l.act != "relu":
+                mlp["act"] = l.act
+            out.append({"type": l.kind, "mixer": mixer, "mlp": mlp})
         return {"architecture": self.ARCHITECTURE, "embedding": {"scale": self.embed_scale}, "layers": out,
                 "norm": {"eps": self.norm_eps}, "vocab": self.vocab_size, "width": self.hidden_size}
 

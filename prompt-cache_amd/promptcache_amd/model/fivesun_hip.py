@@ -66,6 +66,8 @@ def rotary_frequencies(base: float, dims: int, factor: float = 1.0, original: fl
 
 class FivesunHIP(SlotModel):
     GRAPH_MAX_ROWS = 64
+    SEGMENT = int(os.environ.get("PC_FS_SEGMENT", "64"))    # a step that brings a request more tokens than this runs its mLSTM layers segment-parallel
+    MAX_SEGMENTS = 128      # (segments grow beyond SEGMENT tokens rather than exceed this many per request)
 
     def __init__(self, shape: FivesunShape, weights: Dict[str, torch.Tensor], device="cuda:0", dtype=torch.bfloat16,
                  decode_headroom: int = 256):
@@ -214,16 +216,33 @@ class FivesunHIP(SlotModel):
         # rows of the per-head projections: bucket h holds (token, head h) for every token; perm[h * T + t] = t * H + h
         perms = [np.concatenate([(np.arange(T, dtype=np.int32) * H + h) for h in range(H)] + [np.arange(H + 1, dtype=np.int32) * T])
                  for H in self._perm_heads]
+        # segments of the matrix memories' prefill (only when some request brings more than SEGMENT tokens)
+        seg_a = seg_c = chains = np.zeros((0, 4), np.int32)
+        seg_end = np.zeros(0, np.int32)
+        if max(counts) > self.SEGMENT and any(l.kind == "mlstm" for l in self.config.layers):
+            seg = max(self.SEGMENT, -(-max(counts) // self.MAX_SEGMENTS))
+            sa, ch = [], []
+            for b, (s, st, c) in enumerate(zip(slots, starts, counts)):
+                ch.append((s, st, len(sa), -(-c // seg)))
+                sa += [(len(sa) + k, 0, min(seg, c - q), int(row0[b]) + q) for k, q in enumerate(range(0, c, seg))]
+            seg_a = np.asarray(sa, dtype=np.int32)
+            seg_c = seg_a.copy()
+            seg_c[:, 1] = 1                                 # the second pass starts every segment from a state that was put there
+            chains = np.asarray(ch, dtype=np.int32)
+            seg_end = np.full(len(sa), -1, dtype=np.int32)  # a request's last segment leaves the slot's new state
+            seg_end[chains[:, 2] + chains[:, 3] - 1] = chains[:, 0]
         offs = np.stack([row_slot * (g * arena.cap * d) + row_pos * d for g, d in self._sigs] +
                         [row_slot * (g * d * arena.cap) + row_pos for g, d in self._vsigs]) if self._sigs else np.zeros((0, T), np.int64)
         # one block: int32 tables, then int64 cache offsets
-        parts32 = [ids, row_pos.astype(np.int32), reqs.reshape(-1), tiles.reshape(-1), want_rows] + perms
+        parts32 = [ids, row_pos.astype(np.int32), reqs.reshape(-1), tiles.reshape(-1), want_rows, seg_a.reshape(-1), seg_c.reshape(-1),
+                   chains.reshape(-1), seg_end] + perms
         n32 = sum(p.size for p in parts32)
         o64 = (n32 * 4 + 7) // 8 * 8
         blob = np.empty(o64 + offs.size * 8 + 8, dtype=np.uint8)
         blob[:n32 * 4].view(np.int32)[:] = np.concatenate(parts32)
         blob[o64:o64 + offs.size * 8].view(np.int64)[:] = offs.reshape(-1)
-        dims = dict(T=T, R=R, n_tiles=tiles.shape[0], n_want=int(want_rows.size), n32=n32, o64=o64)
+        dims = dict(T=T, R=R, n_tiles=tiles.shape[0], n_want=int(want_rows.size), n32=n32, o64=o64, n_seg=seg_a.shape[0],
+                    n_chains=chains.shape[0])
         res = self._decode_graphed(arena, blob, dims) if graphed else None
         if res is None:
             dblob = torch.from_numpy(blob).to(dev)
@@ -239,7 +258,10 @@ class FivesunHIP(SlotModel):
         T, R, nt, nw = d["T"], d["R"], d["n_tiles"], d["n_want"]
         i32 = dblob[:d["n32"] * 4].view(torch.int32)
         at, out = 0, {}
-        for name, n in [("ids", T), ("pos", T), ("reqs", 4 * R), ("tiles", 4 * nt), ("want", nw)] + \
+        ns = d["n_seg"]
+        out["n_seg"], out["n_chains"] = ns, d["n_chains"]
+        for name, n in [("ids", T), ("pos", T), ("reqs", 4 * R), ("tiles", 4 * nt), ("want", nw), ("seg_a", 4 * ns), ("seg_c", 4 * ns),
+                        ("chains", 4 * d["n_chains"]), ("seg_end", ns)] + \
                        [(("perm", H), T * H + H + 1) for H in self._perm_heads]:
             out[name] = i32[at:at + n]
             at += n
@@ -362,8 +384,18 @@ class FivesunHIP(SlotModel):
         HD, HV = H * D, H * Dv
         P, N = self._project_in(lw, h, T)
         o = self._mat("mix_o32", T, HV, torch.float32)
-        B.mlstm(P, P[:, HD:], P[:, 2 * HD:], P[:, 2 * HD + HV:], P[:, 2 * HD + HV + H:], N, tb["reqs"], R, arena.states[i][0], H, D, Dv,
-                D ** -0.5, l.gate_cap, o)
+        cols = (P, P[:, HD:], P[:, 2 * HD:], P[:, 2 * HD + HV:], P[:, 2 * HD + HV + H:], N)
+        state, ns = arena.states[i][0], tb["n_seg"]
+        if ns:
+            # every segment from nothing (only the states move), the segments chained, then every segment from its start state
+            rec = B.mlstm_state_floats(H, D, Dv)
+            local, start = self._mat("seg_local", ns, rec, torch.float32), self._mat("seg_start", ns, rec, torch.float32)
+            fsum = self._mat("seg_logf", ns, H, torch.float32)
+            B.mlstm(*cols, tb["seg_a"], ns, local, H, D, Dv, D ** -0.5, l.gate_cap, None, from_nothing=True, log_f_sum=fsum)
+            B.mlstm_chain(local, fsum, start, state, tb["chains"], tb["n_chains"], H, D, Dv)
+            B.mlstm(*cols, tb["seg_c"], ns, start, H, D, Dv, D ** -0.5, l.gate_cap, o, end_slots=tb["seg_end"], end_state=state)
+        else:
+            B.mlstm(*cols, tb["reqs"], R, state, H, D, Dv, D ** -0.5, l.gate_cap, o)
         on = self._mat("mix_gated", T, HV, self.dtype)
         B.gated_norm(o, lw["gain"], P[:, 2 * HD + HV + 2 * H:], N, on, self.config.norm_eps, T, group=Dv)
         B.linear(on, lw["wo"], y, M=T)

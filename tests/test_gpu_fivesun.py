@@ -383,6 +383,48 @@ def test_matrix_memory_alone(dtype, H, D, Dv, cap_):
     assert rel(S[:, -1], st3[2]) < 1e-6
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,D,Dv", [(2, 16, 24), (1, 100, 70), (3, 200, 10)])
+def test_matrix_memory_in_segments_equals_token_by_token(dtype, H, D, Dv):
+    """Two requests -- one continues from a state, one starts at position 0 on a slot that holds junk -- cut into segments of
+    unequal lengths that start from nothing, are chained and run again from their start states: outputs and final states equal
+    those of one pass over each request."""
+    b = B()
+    n, cap_ = [75, 41], 5.0
+    T = sum(n)
+    N = 2 * H * D + H * Dv + 2 * H
+    P = rnd(T, N, dtype=dtype, seed=1)
+    P[:, 2 * H * D + H * Dv + H:] += 2.0
+    rec = b.mlstm_state_floats(H, D, Dv)
+    state0 = rnd(3, rec, seed=2)
+    state0.view(3, H, -1)[:, :, -1] = 0.7                      # (a running maximum the first request resumes from)
+    cols = (P, P[:, H * D:], P[:, 2 * H * D:], P[:, 2 * H * D + H * Dv:], P[:, 2 * H * D + H * Dv + H:], N)
+    reqs = [(2, 9, n[0], 0), (0, 0, n[1], n[0])]
+    plain, seg = state0.clone(), state0.clone()
+    want = torch.empty(T, H * Dv, dtype=torch.float32, device=DEV)
+    b.mlstm(*cols, dev_i32(reqs), 2, plain, H, D, Dv, D ** -0.5, cap_, want)
+    cuts = [[16, 1, 30, 28], [40, 1]]
+    sa, chains, at = [], [], 0
+    for (slot, pos, cnt, row), cs in zip(reqs, cuts):
+        chains.append((slot, pos, len(sa), len(cs)))
+        for c in cs:
+            sa.append((len(sa), 0, c, at))
+            at += c
+    ns = len(sa)
+    sc = [(g, 1, c, r) for g, _, c, r in sa]
+    local, start = torch.zeros(ns, rec, device=DEV), torch.zeros(ns, rec, device=DEV)
+    fsum = torch.zeros(ns, H, device=DEV)
+    got = torch.empty_like(want)
+    b.mlstm(*cols, dev_i32(sa), ns, local, H, D, Dv, D ** -0.5, cap_, None, from_nothing=True, log_f_sum=fsum)
+    b.mlstm_chain(local, fsum, start, seg, dev_i32(chains), 2, H, D, Dv)
+    ends = [-1] * ns
+    for slot, _, first, count in chains:
+        ends[first + count - 1] = slot
+    b.mlstm(*cols, dev_i32(sc), ns, start, H, D, Dv, D ** -0.5, cap_, got, end_slots=dev_i32(ends), end_state=seg)
+    assert rel(got, want) < 3e-6
+    assert rel(seg[2], plain[2]) < 3e-6 and rel(seg[0], plain[0]) < 3e-6 and torch.equal(seg[1], state0[1])
+
+
 # =====================================================================================================================================
 # the model through its arena
 # =====================================================================================================================================
