@@ -285,6 +285,8 @@ typedef struct pcb_attn_softmax_args {
     int32_t block;
     const float* sink;
     int32_t gate_per_head;
+    int32_t head_rows; /* 1: every tile has ONE row and there is one key head (Hkv = 1): a workgroup takes 16 heads of that row at once
+                          (the heads read the same keys and values) -- for decoding over a shared latent */
 } pcb_attn_softmax_args;
 int pcb_attn_softmax(const pcb_attn_softmax_args* a, void* stream);
 

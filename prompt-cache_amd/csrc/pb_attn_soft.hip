@@ -9,6 +9,8 @@
 //   O^T = V^T P^T the weights P of a query are exactly what its lanes hold; the k index of this product runs over the 32 keys of
 //                 the block in the order (l >> 4, e) -> key 4 (l >> 4) + e (e < 4), 16 + 4 (l >> 4) + e - 4 (e >= 4), the same for
 //                 both operands, so the permutation cancels.
+// With one key head and tiles of one row each (decoding over a shared latent), head_rows makes the 16 rows of a tile 16 HEADS of that
+// one token instead: the heads read the same keys and values, so one pass over them serves sixteen heads.
 // Scores, maxima, weights and sums are fp32.  bf16: the weights enter the second product as a hi + lo pair of bf16 values (two
 // MFMAs), so they are not rounded to 8 bits; fp32: the fp32 matrix cores take them as they are.
 #include "pb_common.h"
@@ -112,12 +114,15 @@ __global__ __launch_bounds__(64 * AW) void attn_softmax_kernel(pcb_attn_softmax_
     // not be the ones that start last)
     const int32_t* tile = a.tiles + 4 * (gridDim.x - 1 - blockIdx.x);
     const int slot = tile[0], pos0 = tile[1], rows = tile[2], row0 = tile[3];
-    const int h = blockIdx.y, hk = h / (a.H / a.Hkv);
     const int dim = a.dim, vdim = a.vdim;
-    const int last = pos0 + rows - 1;                       // the newest key any query of the tile sees
-    const int qi = c < rows ? c : rows - 1;                 // (lanes past the tile repeat its last query; nothing of theirs is stored)
-    const int qpos = pos0 + qi;
-    const int64_t qrow = row0 + qi;
+    // what the 16 lanes-columns of the tile stand for: its rows (one head, blockIdx.y), or -- head_rows -- 16 heads of its one row
+    const int n_q = a.head_rows ? (a.H - 16 * (int)blockIdx.y < 16 ? a.H - 16 * (int)blockIdx.y : 16) : rows;
+    const int last = pos0 + (a.head_rows ? 0 : rows - 1);   // the newest key any query of the tile sees
+    const int qi = c < n_q ? c : n_q - 1;                   // (lanes past the tile repeat its last query; nothing of theirs is stored)
+    const int h = a.head_rows ? 16 * (int)blockIdx.y + qi : (int)blockIdx.y;
+    const int hk = a.head_rows ? 0 : h / (a.H / a.Hkv);
+    const int qpos = a.head_rows ? pos0 : pos0 + qi;
+    const int64_t qrow = a.head_rows ? row0 : row0 + qi;
     const E* K = (const E*)a.kcache + (int64_t)slot * a.slot_stride + (int64_t)hk * a.head_stride;
     const E* V = (const E*)a.vcache + (int64_t)slot * a.v_slot_stride + (int64_t)hk * a.v_head_stride;
     const E* qp = (const E*)a.q + qrow * a.ldq + (int64_t)h * dim;
@@ -270,7 +275,7 @@ __global__ __launch_bounds__(64 * AW) void attn_softmax_kernel(pcb_attn_softmax_
 #pragma unroll
             for (int r = 0; r < 4; ++r) o[vb][r] += fw * red_o[w][(vb * 4 + r) * 64 + lane];
     }
-    if (c >= rows) return;
+    if (c >= n_q) return;
     if (a.n_splits > 1) {
         float* pp = a.part + ((qrow * a.H + h) * a.n_splits + blockIdx.z) * (int64_t)(vdim + 2);
         if (g == 0) pp[vdim] = mm, pp[vdim + 1] = lt;
@@ -343,7 +348,7 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(pcb_attn_softmax_args a
 
 template <typename E>
 int dispatch(const pcb_attn_softmax_args& a, hipStream_t stream) {
-    const dim3 grid(a.n_tiles, a.H, a.n_splits > 1 ? a.n_splits : 1), block(64 * AW);
+    const dim3 grid(a.n_tiles, a.head_rows ? (a.H + 15) / 16 : a.H, a.n_splits > 1 ? a.n_splits : 1), block(64 * AW);
     const int big = a.dim > a.vdim ? a.dim : a.vdim;
     if (big <= 64)
         hipLaunchKernelGGL((attn_softmax_kernel<E, 2, 4>), grid, block, 0, stream, a);
@@ -372,6 +377,7 @@ PCB_EXPORT int pcb_attn_softmax(const pcb_attn_softmax_args* a, void* stream) {
     PCB_REQUIRE(a->q && a->tiles && a->kcache && a->vcache && a->out &&
                     (!a->gate || a->ldg >= (a->gate_per_head ? (int64_t)a->H : (int64_t)a->H * a->vdim)),
                 PCB_ERR_ARG, "pcb_attn_softmax: null pointer");
+    PCB_REQUIRE(!a->head_rows || a->Hkv == 1, PCB_ERR_ARG, "pcb_attn_softmax: heads as rows need one key head (and tiles of one row)");
     PCB_REQUIRE(a->n_splits <= 1 || (a->part && a->n_splits <= 64), PCB_ERR_ARG, "pcb_attn_softmax: up to 64 runs, with their scratch");
     return a->dtype == PCB_BF16 ? dispatch<pcb::bf16_t>(*a, (hipStream_t)stream) : dispatch<float>(*a, (hipStream_t)stream);
 }

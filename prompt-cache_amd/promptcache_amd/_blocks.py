@@ -73,7 +73,7 @@ class AttnSoftmaxArgs(C.Structure):
                 ("v_slot_stride", _i64), ("v_head_stride", _i64), ("v_stride", _i64), ("v_cols", _i32),
                 ("H", _i32), ("Hkv", _i32), ("dim", _i32), ("vdim", _i32), ("scale", _f32), ("window", _i32),
                 ("gate", _vp), ("ldg", _i64), ("out", _vp), ("ldo", _i64), ("n_splits", _i32), ("part", _vp),
-                ("block", _i32), ("sink", _vp), ("gate_per_head", _i32)]
+                ("block", _i32), ("sink", _vp), ("gate_per_head", _i32), ("head_rows", _i32)]
 
 
 class DecayAttnArgs(C.Structure):
@@ -442,14 +442,15 @@ def attn_softmax(q: torch.Tensor, ldq: int, tiles: torch.Tensor, n_tiles: int, k
                  v_offset: int, v_strides, v_cols: bool, H: int, Hkv: int, dim: int, vdim: int, scale: float, out: torch.Tensor, *,
                  q_scale: Optional[torch.Tensor] = None, window: int = 0, gate: Optional[torch.Tensor] = None, ldg: int = 0,
                  n_splits: int = 1, part: Optional[torch.Tensor] = None, block: int = 0, sink: Optional[torch.Tensor] = None,
-                 gate_per_head: bool = False) -> None:
+                 gate_per_head: bool = False, head_rows: bool = False) -> None:
     """``q``: E rows (row stride ``ldq``, head h at column h * dim); ``kcache`` with ``k_strides`` = (slot, head, row) strides in
     elements; the values start ``v_offset`` elements into ``vcache`` (which may be the same plane) with ``v_strides`` = (slot, head,
     row) strides, or (slot, head, column) strides when ``v_cols`` (a cache kept column by column, columns readable in multiples of
     32 keys); ``gate``: E rows of stride ``ldg``; ``out`` E [rows, H * vdim].  ``n_splits`` > 1: each (tile, head) runs as that many
     workgroups over runs of the keys, merged by a second launch; ``part``: fp32 scratch of ``attn_softmax_part(rows, H, n_splits,
     vdim)`` floats.  ``block`` > 0: a key is seen only inside the query's own block of that many positions; ``sink`` fp32 [H]: one
-    more exp(sink[h]) in the denominator; ``gate_per_head``: the gate has one column per head."""
+    more exp(sink[h]) in the denominator; ``gate_per_head``: the gate has one column per head; ``head_rows``: every tile has one row and
+    there is one key head -- a workgroup then serves 16 heads of the row at once."""
     _want(tiles, torch.int32, "attn_softmax tiles"); _want(q_scale, torch.float32, "attn_softmax q_scale")
     _want(sink, torch.float32, "attn_softmax sink")
     assert sink is None or sink.numel() == H
@@ -460,7 +461,7 @@ def attn_softmax(q: torch.Tensor, ldq: int, tiles: torch.Tensor, n_tiles: int, k
     a = AttnSoftmaxArgs(C.sizeof(AttnSoftmaxArgs), _code(q), _p(q), ldq, _p(q_scale), _p(tiles), n_tiles, _p(kcache),
                         vcache.data_ptr() + v_offset * es, int(k_strides[0]), int(k_strides[1]), int(k_strides[2]), int(v_strides[0]),
                         int(v_strides[1]), int(v_strides[2]), int(v_cols), H, Hkv, dim, vdim, float(scale), int(window), _p(gate), ldg,
-                        _p(out), out.shape[-1], int(n_splits), _p(part), int(block), _p(sink), int(gate_per_head))
+                        _p(out), out.shape[-1], int(n_splits), _p(part), int(block), _p(sink), int(gate_per_head), int(head_rows))
     if n_splits > 1:
         _want(part, torch.float32, "attn_softmax part")
         assert part.numel() >= attn_softmax_part(out.shape[0], H, n_splits, vdim)

@@ -368,10 +368,11 @@ class FivesunHIP(SlotModel):
         B.linear(qn.view(T * H, D), lw["w_abs"], qa.view(T * H, CR), M=T * H, row_src=rows, row_dst=rows, group_off=goff, n_groups=H,
                  ldy=CR)
         ol = self._mat("mix_out", T, H * C, E)
-        splits = self._splits(arena, n_tiles, H)
+        one_each = T == R                                    # one token per request: 16 heads share a pass over the slot's rows
+        splits = self._splits(arena, n_tiles, -(-H // 16) if one_each else H)
         part = self._scratch("attn_part", B.attn_softmax_part(T, H, splits, C), torch.float32) if splits > 1 else None
         B.attn_softmax(qa, H * CR, tb["tiles"], n_tiles, plane, (arena.slot_stride(i), 0, CR), plane, 0, (arena.slot_stride(i), 0, CR),
-                       False, H, 1, CR, C, l.scale, ol, window=l.mask, n_splits=splits, part=part)
+                       False, H, 1, CR, C, l.scale, ol, window=l.mask, n_splits=splits, part=part, head_rows=one_each)
         ov = self._mat("mix_o32", T, HV, torch.float32)
         B.linear(ol.view(T * H, C), lw["w_uv"], ov.view(T * H, Dv), M=T * H, row_src=rows, row_dst=rows, group_off=goff, n_groups=H)
         og = self._mat("mix_gated", T, HV, E)

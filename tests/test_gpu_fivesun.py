@@ -242,7 +242,7 @@ def test_head_preparation_norm_blend_rotation_and_destinations(dtype):
     assert float(kplane.float().abs().sum(dim=(1, 3)).cpu()[untouched].sum()) == 0.0
 
 
-def _attend(dtype, q, keys, vals, qpos, H, G, scale, *, window=0, block=0, sink=None, gate=None, splits=1, cols=True):
+def _attend(dtype, q, keys, vals, qpos, H, G, scale, *, window=0, block=0, sink=None, gate=None, splits=1, cols=True, head_rows=False):
     """q [n, H, D] at positions qpos of ONE sequence whose keys [m, G, D] / values [m, G, Dv] sit at positions 0 .. m-1."""
     n, m, D, Dv = q.shape[0], keys.shape[0], q.shape[2], vals.shape[2]
     cap = -(-m // 32) * 32
@@ -260,7 +260,7 @@ def _attend(dtype, q, keys, vals, qpos, H, G, scale, *, window=0, block=0, sink=
     tiles, at = [], 0
     while at < n:
         run = 1
-        while at + run < n and run < 16 and qpos[at + run] == qpos[at] + run:
+        while at + run < n and run < 16 and qpos[at + run] == qpos[at] + run and not head_rows:
             run += 1
         tiles.append((1, qpos[at], run, at))
         at += run
@@ -268,7 +268,7 @@ def _attend(dtype, q, keys, vals, qpos, H, G, scale, *, window=0, block=0, sink=
     part = torch.empty(B().attn_softmax_part(n, H, splits, Dv), dtype=torch.float32, device=DEV) if splits > 1 else None
     B().attn_softmax(q.reshape(n, H * D).contiguous(), H * D, dev_i32(tiles), len(tiles), kplane, (G * cap * D, cap * D, D), vplane, 0, vstr, cols,
                      H, G, D, Dv, scale, out, window=window, block=block, sink=sink, gate=gate, ldg=H if gate is not None else 0,
-                     gate_per_head=gate is not None, n_splits=splits, part=part)
+                     gate_per_head=gate is not None, n_splits=splits, part=part, head_rows=head_rows)
     return out.view(n, H, Dv)
 
 
@@ -295,6 +295,25 @@ def test_attention_blocks_sinks_and_head_gates(dtype, splits, D, Dv, cols):
     got = _attend(dtype, q, keys, vals, qpos, H, G, 0.3, block=block, sink=sink, gate=gate, splits=splits, cols=cols)
     want = _attend_oracle(q, keys, vals, qpos, H, G, 0.3, lambda i, j: O.sees_block(i, j, block), sink, gate)
     assert rel(got, want) < tol(dtype, 1e-5, 1e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("splits", [1, 4])
+@pytest.mark.parametrize("H", [20, 3])
+def test_sixteen_heads_of_one_token_share_a_pass_over_one_key_head(dtype, splits, H):
+    """Single decoded rows over ONE key head whose values are the first columns of the key rows themselves (a shared latent):
+    heads as the rows of a tile, a full block of 16 and a partial one, with a window."""
+    D, Dv, m, window = 40, 24, 200, 90
+    keys = rnd(m, 1, D, dtype=dtype, seed=1)
+    vals = keys[:, :, :Dv].contiguous()
+    qpos = [0, 5, 89, 90, 91, 150, 199]
+    q = rnd(len(qpos), H, D, dtype=dtype, seed=3)
+    sink = rnd(H, seed=4)
+    got = _attend(dtype, q, keys, vals, qpos, H, 1, 0.2, window=window, sink=sink, splits=splits, cols=False, head_rows=True)
+    want = _attend_oracle(q, keys, vals, qpos, H, 1, 0.2, lambda i, j: O.sees_window(i, j, window), sink)
+    assert rel(got, want) < tol(dtype, 1e-5, 1e-2)
+    same = _attend(dtype, q, keys, vals, qpos, H, 1, 0.2, window=window, sink=sink, splits=splits, cols=False)
+    assert rel(got, same) < tol(dtype, 1e-6, 1e-6)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
