@@ -591,6 +591,30 @@ def test_greedy_generation_through_the_batch_engine(dtype):
             seq.append(tok)
 
 
+def test_single_request_engine_and_the_adapters_call():
+    """GenerationEngine drives the model through the adapters' ``model(input_ids, past_key_values)`` call; a padded batch through
+    that call gives each row its own logits."""
+    from promptcache_amd import BatchEngine, GenerationEngine, GenerationParameters
+    from promptcache_amd.model import Fivesun
+    s = shape_mixed()
+    w = W.make_fivesun_weights(s, seed=21)
+    lm = Fivesun(shape=s, weights=w, device=DEV, dtype=torch.float32)
+    prompts = [toks(13, s.vocab_size, 30), toks(5, s.vocab_size, 31)]
+    params = GenerationParameters(temperature=0.0, max_new_tokens=6, stop_token_ids=[])
+    want = BatchEngine(lm).generate(prompts, params)
+    out = None
+    for out in GenerationEngine(lm).generate(prompts[0], list(range(13)), params):
+        pass
+    assert out is not None and lm.decode(want[0]) == out.new_text
+    ids, mask = torch.zeros((2, 13), dtype=torch.long), torch.zeros((2, 13), dtype=torch.long)
+    ids[0, :13], mask[0, :13] = torch.tensor(prompts[0]), 1
+    ids[1, :5], mask[1, :5] = torch.tensor(prompts[1]), 1
+    res = lm(input_ids=ids, attention_mask=mask, past_key_values=None, use_cache=True)
+    p6 = O.to_f64(w)
+    assert rel(res.logits[0], O.forward(s, p6, prompts[0])[0]) < 3e-5 and rel(res.logits[1, :5], O.forward(s, p6, prompts[1])[0]) < 3e-5
+    assert int(res.logits[0, 12].argmax()) == want[0][0] and int(res.logits[1, 4].argmax()) == want[1][0]
+
+
 def test_checkpoint_directory_command_line_and_trace_runner(tmp_path):
     """config.json + model.safetensors written from a shape, found by the registry, and replayed by bin/trace_run in both formats."""
     from safetensors.torch import save_file
