@@ -618,13 +618,13 @@ class FivesunShape:
         for kind in pattern:
             if kind == "attention":
                 lay = FivesunLayer(kind, heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, scale=dim ** -0.5, mask=chunk,
-                                   rot_base=500000.0, rot_dims=dim, rot_factor=2.0, v_mix=True)
+                                   rot_base=1000000.0, rot_dims=dim, rot_factor=4.0, v_mix=True)
             elif kind == "latent_attention":
                 lay = FivesunLayer(kind, heads=heads, kv_heads=1, dim=dim, vdim=dim, kv_rank=kv_rank or 4 * dim, rot_dim=rot_dim,
-                                   rot_dims=rot_dim, scale=(dim + rot_dim) ** -0.5, mask=window, rot_base=250000.0, rot_factor=2.0,
-                                   yarn_original=2048.0)
+                                   rot_dims=rot_dim, scale=(dim + rot_dim) ** -0.5, mask=window, rot_base=10000.0, rot_factor=8.0,
+                                   yarn_original=4096.0)
             else:
-                lay = FivesunLayer("mlstm", heads=heads, kv_heads=heads, dim=dim, vdim=dim, gate_cap=15.0)
+                lay = FivesunLayer("mlstm", heads=heads, kv_heads=heads, dim=dim, vdim=dim, gate_cap=10.0)
             lay.ff = ff
             layers.append(lay)
         return cls(vocab_size=vocab, hidden_size=width, norm_eps=1e-6, layers=layers, embed_scale=width ** 0.5, name=name)
