@@ -591,6 +591,52 @@ def test_greedy_generation_through_the_batch_engine(dtype):
             seq.append(tok)
 
 
+def random_shape(rng):
+    """Sizes, layer order, masks, rotated parts and constants drawn at random (blended values share one shape, as they must)."""
+    width = rng.choice([64, 72, 96, 160, 200, 256])
+    G, Dv = rng.choice([1, 2, 3, 4]), rng.choice([16, 24, 40, 64, 72])
+    layers = []
+    for _ in range(rng.randrange(2, 6)):
+        kind, ff = rng.choice(["attention", "latent_attention", "mlstm"]), rng.choice([0, 32, 56, width, 2 * width])
+        if kind == "attention":
+            vm = rng.random() < 0.6
+            g = G if vm else rng.choice([1, 2, 4])
+            dim = rng.choice([16, 24, 48, 64, 96, 160])
+            layers.append(att(g * rng.choice([1, 2, 3, 4]), g, dim, Dv if vm else rng.choice([16, 40, 128]), mask=rng.choice([0, 1, 7, 32, 50, 100]),
+                              rot_dims=rng.choice([dim, dim // 4 * 2, 0]), v_mix=vm, ff=ff, factor=rng.choice([1.0, 2.5]), scale=0.7 * dim ** -0.5))
+        elif kind == "latent_attention":
+            layers.append(lat(rng.choice([1, 2, 6, 12, 20]), rng.choice([16, 32, 48, 96]), rng.choice([0, 4, 8, 32, 64]), rng.choice([16, 32, 80]),
+                              rng.choice([16, 40, 96, 200, 256]), mask=rng.choice([0, 1, 5, 33, 96]), ff=ff, original=rng.choice([0.0, 64.0, 1000.0]),
+                              factor=rng.choice([2.0, 8.0]), fast=rng.choice([32.0, 8.0]), slow=rng.choice([1.0, 2.0])))
+        else:
+            layers.append(mls(rng.choice([1, 2, 4, 8]), rng.choice([8, 16, 48, 100, 192]), rng.choice([8, 16, 48, 130]), cap=rng.choice([0.0, 5.0, 11.0]), ff=ff))
+    return FivesunShape(vocab_size=rng.randrange(50, 900), hidden_size=width, norm_eps=rng.choice([1e-5, 1e-6]),
+                        embed_scale=rng.choice([1.0, width ** 0.5]), layers=layers)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_configurations_whole_decoded_and_in_company(seed):
+    import random
+    from promptcache_amd.model.fivesun_hip import FivesunHIP
+    rng = random.Random(1000 + seed)
+    s = FivesunShape.from_config(json.loads(json.dumps(random_shape(rng).to_config())))
+    w = W.make_fivesun_weights(s, seed=seed)
+    n = rng.randrange(90, 260)
+    a, b_ = toks(n, s.vocab_size, seed), toks(rng.randrange(1, 70), s.vocab_size, seed + 1)
+    want_a, want_b = oracle_logits(s, w, a)[0], oracle_logits(s, w, b_)[0]
+    for dtype in DTYPES:
+        m = FivesunHIP(s, w, device=DEV, dtype=dtype)
+        t = tol(dtype, 5e-5, 0.15)
+        assert rel(run_alone(m, a), want_a) < t, s.to_config()
+        ar = m.new_arena(1, 16)
+        sa, sb = ar.alloc(), ar.alloc()
+        cut = n - 20
+        out = [m.forward_rows(ar, [sb, sa], [b_, a[:cut]], [list(range(len(b_))), list(range(cut))])]
+        out += [m.forward_rows(ar, [sa], [[t_]], [[0]]) for t_ in a[cut:]]
+        got = torch.cat(out)
+        assert rel(got[len(b_):], want_a) < t and rel(got[:len(b_)], want_b) < t, s.to_config()
+
+
 def test_single_request_engine_and_the_adapters_call():
     """GenerationEngine drives the model through the adapters' ``model(input_ids, past_key_values)`` call; a padded batch through
     that call gives each row its own logits."""
