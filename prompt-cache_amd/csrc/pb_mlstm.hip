@@ -24,7 +24,8 @@ __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.0f) - 
 
 constexpr int TB = 8;          // tokens per staged block
 
-template <typename E, int DPT>
+// OUT false: only the states move (the first pass over segments) -- no products with q, no partial sums, no barrier per token
+template <typename E, int DPT, bool OUT>
 __global__ __launch_bounds__(256) void mlstm_kernel(pcb_mlstm_args a) {
     constexpr int DM = 4 * DPT;                 // key rows the workgroup can hold (>= dim)
     constexpr int QN = TB * DM / 256;           // q (and k) elements a thread fetches per block
@@ -65,7 +66,7 @@ __global__ __launch_bounds__(256) void mlstm_kernel(pcb_mlstm_args a) {
         for (int i = 0; i < QN; ++i) {
             const int e = tid + 256 * i, tt = e / DM, d = e % DM;
             const bool ok = d < dim && t0 + tt < count;
-            rq_[i] = ok ? to_f32(q[(int64_t)(t0 + tt) * a.ldq + d]) * a.q_scale : 0.0f;
+            rq_[i] = (OUT && ok) ? to_f32(q[(int64_t)(t0 + tt) * a.ldq + d]) * a.q_scale : 0.0f;
             rk_[i] = ok ? to_f32(k[(int64_t)(t0 + tt) * a.ldk + d]) : 0.0f;
         }
 #pragma unroll
@@ -82,7 +83,7 @@ __global__ __launch_bounds__(256) void mlstm_kernel(pcb_mlstm_args a) {
 #pragma unroll
         for (int i = 0; i < QN; ++i) {
             const int e = tid + 256 * i;
-            qs[b][e / DM][e % DM] = rq_[i];
+            if (OUT) qs[b][e / DM][e % DM] = rq_[i];
             ks[b][e / DM][e % DM] = rk_[i];
         }
 #pragma unroll
@@ -116,21 +117,24 @@ __global__ __launch_bounds__(256) void mlstm_kernel(pcb_mlstm_args a) {
             const float4* q4 = reinterpret_cast<const float4*>(&qs[b][tt][p * DPT]);
 #pragma unroll
             for (int i4 = 0; i4 < DPT / 4; ++i4) {
-                const float4 kk = k4[i4], qq = q4[i4];
+                const float4 kk = k4[i4], qq = OUT ? q4[i4] : float4{0.f, 0.f, 0.f, 0.f};
                 const float kd[4] = {kk.x, kk.y, kk.z, kk.w}, qd[4] = {qq.x, qq.y, qq.z, qq.w};
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int i = 4 * i4 + e;
                     S[i] = keep * S[i] + kd[e] * tv;
                     nv[i] = keep * nv[i] + take * kd[e];
-                    acc += S[i] * qd[e];
-                    accn += nv[i] * qd[e];
+                    if (OUT) {
+                        acc += S[i] * qd[e];
+                        accn += nv[i] * qd[e];
+                    }
                 }
             }
+            if (!OUT) continue;
             part_o[pb][p][lane] = acc;
             if (lane == 0) part_n[pb][p] = accn;
             __syncthreads();
-            if (p == 0 && col && a.out) {
+            if (p == 0 && col) {
                 const float num = (part_o[pb][0][lane] + part_o[pb][1][lane]) + (part_o[pb][2][lane] + part_o[pb][3][lane]);
                 const float nq_dot = (part_n[pb][0] + part_n[pb][1]) + (part_n[pb][2] + part_n[pb][3]);
                 const float den = fmaxf(fabsf(nq_dot), expf(-m_new)) + 1e-6f;
@@ -192,12 +196,21 @@ __global__ __launch_bounds__(256) void mlstm_chain_kernel(const float* __restric
 template <typename E>
 int dispatch(const pcb_mlstm_args& a, hipStream_t stream) {
     const dim3 grid(a.n_reqs, a.H, pcb_ceil_div(a.vdim, 64)), block(256);
-    if (a.dim <= 64)
-        hipLaunchKernelGGL((mlstm_kernel<E, 16>), grid, block, 0, stream, a);
-    else if (a.dim <= 128)
-        hipLaunchKernelGGL((mlstm_kernel<E, 32>), grid, block, 0, stream, a);
-    else
-        hipLaunchKernelGGL((mlstm_kernel<E, 64>), grid, block, 0, stream, a);
+    if (a.out) {
+        if (a.dim <= 64)
+            hipLaunchKernelGGL((mlstm_kernel<E, 16, true>), grid, block, 0, stream, a);
+        else if (a.dim <= 128)
+            hipLaunchKernelGGL((mlstm_kernel<E, 32, true>), grid, block, 0, stream, a);
+        else
+            hipLaunchKernelGGL((mlstm_kernel<E, 64, true>), grid, block, 0, stream, a);
+    } else {
+        if (a.dim <= 64)
+            hipLaunchKernelGGL((mlstm_kernel<E, 16, false>), grid, block, 0, stream, a);
+        else if (a.dim <= 128)
+            hipLaunchKernelGGL((mlstm_kernel<E, 32, false>), grid, block, 0, stream, a);
+        else
+            hipLaunchKernelGGL((mlstm_kernel<E, 64, false>), grid, block, 0, stream, a);
+    }
     return pcb_check_launch("mlstm_kernel");
 }
 
