@@ -16,7 +16,7 @@
 extern "C" {
 #endif
 
-#define PCB_ABI_VERSION 3
+#define PCB_ABI_VERSION 4
 #define PCB_OK 0
 #define PCB_ERR_ARG (-2001)
 #define PCB_ERR_HIP_BASE (-3000)
@@ -73,7 +73,7 @@ int pcb_mix_norm(const pcb_mix_norm_args* a, void* stream);
 #define PCB_EPI_STORE 0
 #define PCB_EPI_SILU_MUL 1
 #define PCB_EPI_SCALE_ADD 2
-/* element-wise function of a STORE epilogue: z, z sigmoid(z), sigmoid(z), max(z, 0)^2, ln(1 + e^z), cap tanh(z / cap) */
+/* element-wise function of a STORE epilogue: z, z sigmoid(z), sigmoid(z), max(z, 0)^2, ln(1 + e^z), cap tanh(z / cap), ... */
 #define PCB_ACT_NONE 0
 #define PCB_ACT_SILU 1
 #define PCB_ACT_SIGMOID 2
@@ -82,6 +82,8 @@ int pcb_mix_norm(const pcb_mix_norm_args* a, void* stream);
 #define PCB_ACT_SOFTCAP 5
 #define PCB_ACT_RELU 6      /* max(z, 0) */
 #define PCB_ACT_GELU_TANH 7 /* 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))) */
+#define PCB_ACT_LOGSIGMOID 8 /* act_param * ln(sigmoid(z)): the logarithm of a decay sigmoid(z)^act_param */
+#define PCB_ACT_SCALE 9      /* act_param * z */
 typedef struct pcb_linear_args {
     uint32_t struct_bytes;
     int32_t dtype;
@@ -119,7 +121,7 @@ typedef struct pcb_linear_args {
     int32_t act;       /* PCB_ACT_*: STORE only, applied to acc + bias before the store (not to the columns split off to y2 / y3) */
     int32_t act_split; /* > 0: columns n >= act_split take act2 instead of act */
     int32_t act2;
-    float act_param;   /* PCB_ACT_SOFTCAP: the cap */
+    float act_param;   /* PCB_ACT_SOFTCAP: the cap; PCB_ACT_LOGSIGMOID, PCB_ACT_SCALE: the factor (it serves act and act2 alike) */
     const void* bias2; /* [N] E, may be null: the second product's bias of the gated epilogue */
 } pcb_linear_args;
 int pcb_linear(const pcb_linear_args* a, void* stream);
@@ -223,9 +225,12 @@ int pcb_hyper_norm(const pcb_hyper_norm_args* a, void* stream);
 /* out[r][c] = E( (gain ? x[r][c] / sqrt(mean x[r]^2 + eps) * gain[c] : x[r][c]) * (gate ? gate[r][c] : 1) ), x fp32 [n_rows][ldx],
  * gate E [n_rows][ldg], out E [n_rows][ldo]: a unit norm with an element-wise gate.  The mean runs over all `cols` columns
  * (group_cols <= 0: one norm over all heads' outputs) or over each run of group_cols columns by itself (a norm per head;
- * group_cols divides cols; then the norm is taken with or without a gain). */
+ * group_cols divides cols; then the norm is taken with or without a gain).
+ * skip (E [n_rows][lds], optional): x[r][c] + skip_w[c / skip_group] * skip[r][c] stands for x[r][c] (a skip path with one weight per
+ * head).  gate_first: the gate is applied BEFORE the norm, out = norm(x * gate) * gain. */
 int pcb_gated_norm(const float* x, int64_t ldx, const float* gain, const void* gate, int64_t ldg, void* out, int64_t ldo,
-                   int32_t dtype, float eps, int32_t n_rows, int32_t cols, int32_t group_cols, void* stream);
+                   int32_t dtype, float eps, int32_t n_rows, int32_t cols, int32_t group_cols, int32_t gate_first, const void* skip,
+                   int64_t lds, const float* skip_w, int32_t skip_group, void* stream);
 
 /* Router choice over n_out outputs per row (logits fp32 [n_rows][n_out]):
  *   score s = score_fn == PCB_SCORE_SOFTMAX ? softmax(logits) : sigmoid(logits);  choice score = s + correction (if given)
@@ -253,7 +258,7 @@ int pcb_moe_mix(const float* pair_out, const int32_t* expert, const float* weigh
  * interleave in one plane), or column by column (v_cols = 1: column c of key j at vcache + s * v_slot_stride + g * v_head_stride +
  * c * v_stride + j; every column must be readable up to the next multiple of 32 keys, and v_stride a multiple of 8), which lets
  * the value operand of the matrix cores be read with wide loads.  The cache already holds the queries' own keys and values.  score = q_scale[row] * scale * q.k (q_scale null: 1); key j is seen by the query at position i iff j <= i and
- * (window <= 0 or i - j < window) and (block <= 0 or floor(i / block) == floor(j / block): blocks of positions counted from 0, a
+ * (window <= 0 or i - j < window or j < keep_first) and (block <= 0 or floor(i / block) == floor(j / block): blocks of positions counted from 0, a
  * key is seen inside the query's own block only).  sink (fp32 [H], optional): the softmax denominator of head h also holds
  * exp(sink[h]) -- a term without key or value, not scaled.  The result (E [rows][ldo], head h at column h * vdim) is multiplied by
  * a gate when given (E, row stride ldg): element-wise gate[row][h * vdim + c], or one number per head gate[row][h] when
@@ -287,6 +292,8 @@ typedef struct pcb_attn_softmax_args {
     int32_t gate_per_head;
     int32_t head_rows; /* 1: every tile has ONE row and there is one key head (Hkv = 1): a workgroup takes 16 heads of that row at once
                           (the heads read the same keys and values) -- for decoding over a shared latent */
+    int32_t keep_first; /* > 0 (with a window): keys at positions < keep_first stay visible to every later query, at their true
+                           positions (the sequence's first tokens are kept behind the sliding window) */
 } pcb_attn_softmax_args;
 int pcb_attn_softmax(const pcb_attn_softmax_args* a, void* stream);
 
@@ -374,6 +381,8 @@ int pcb_state_chain(const float* local, float* start, float* state, int64_t slot
  *   write (y given):  t = y[src] * (gate ? gate[src] : 1);  x[src] += post_gain ? t / sqrt(mean(t^2) + eps) * post_gain : t
  *                     (with `rows` the sum is used but not written back)
  *   read (out given): out[r] = x[src] / sqrt(mean(x[src]^2) + eps) * gain as E;  x_out[r] = x[src] (fp32) if given
+ *                     layer_norm: out[r] = (x - mean(x)) / sqrt(mean((x - mean(x))^2) + eps) * gain + bias instead
+ * y_scale: the sublayer's result enters as y_scale * y (after gate and post norm; 1 = as it is).
  * src = rows ? rows[r] : r.  y fp32 [..][width]; gate E rows of stride ldg; x fp32 [..][width].  width <= 16384. */
 typedef struct pcb_post_norm_args {
     uint32_t struct_bytes;
@@ -390,6 +399,9 @@ typedef struct pcb_post_norm_args {
     float eps;
     int32_t n_rows;
     int32_t width;
+    float y_scale;
+    int32_t layer_norm;
+    const float* bias; /* [width] fp32, layer_norm only (null: none) */
 } pcb_post_norm_args;
 int pcb_post_norm(const pcb_post_norm_args* a, void* stream);
 
@@ -482,6 +494,42 @@ int pcb_mlstm(const pcb_mlstm_args* a, void* stream);
  * local, start: fp32 [segments][H][record]; state is only read. */
 int pcb_mlstm_chain(const float* local, const float* log_f_sum, float* start, const float* state, int64_t slot_stride, const int32_t* chains,
                     int32_t n_chains, int32_t H, int32_t dim, int32_t vdim, void* stream);
+
+/* Linear attention whose decay changes from token to token, with a matrix state per (slot, head):
+ *   S_t = diag(exp(l_t)) S_(t-1) + k_t (s_t v_t)^T,   o_t = S_t^T (q_scale q_t)        (S: [dim][vdim], fp32, zero before position 0)
+ * l_t = ld_coef[h] * ld[row][h * dcols + (dcols == 1 ? 0 : d)] is the log decay of key row d (ld_coef null: 1): dcols = dim gives every
+ * key channel its own decay (gated linear attention), dcols = 1 one decay per head and token (the matrix form of a selective
+ * scan with scalar decays: k = B, q = C, v = x, s = the step size, l = -rate * step size).  s_t = v_scale[row][h] (null: 1).
+ * q, k: E rows with head h / (H / Hk) at column (h / (H / Hk)) * dim (Hk heads of queries and keys serve H heads of values);
+ * v: head h at column h * vdim; ld, v_scale: fp32 rows; out fp32 [rows][ldo].  request r = {slot, first position, tokens, first
+ * flat row} as in pcb_decay_attn; state fp32 [slots][H][dim][vdim].  Decays, step sizes and every product that feeds a state are
+ * fp32.  dim <= 256.
+ * out null: only the states move (the first pass of a segmented prefill); ld_sum (fp32 [n_reqs][H * dcols], optional) receives each
+ * request's sum of log decays, which is what pcb_state_chain needs (coef = 1, group = vdim or dim * vdim). */
+typedef struct pcb_gla_args {
+    uint32_t struct_bytes;
+    int32_t dtype;
+    const void* q;
+    const void* k;
+    const void* v;
+    int64_t ldq, ldk, ldv;
+    const float* ld;
+    int64_t ldld;
+    int32_t dcols;
+    const float* ld_coef;
+    const float* v_scale;
+    int64_t ldvs;
+    const int32_t* reqs;
+    int32_t n_reqs;
+    float* state;
+    int64_t slot_stride;
+    int32_t H, Hk, dim, vdim;
+    float q_scale;
+    float* out;
+    int64_t ldo;
+    float* ld_sum;
+} pcb_gla_args;
+int pcb_gla(const pcb_gla_args* a, void* stream);
 
 #ifdef __cplusplus
 }

@@ -136,8 +136,10 @@ __global__ __launch_bounds__(64 * AW) void attn_softmax_kernel(pcb_attn_softmax_
     const float sc = a.scale * (a.q_scale ? a.q_scale[qrow] : 1.0f) * 1.44269504088896f;
     const float NEG = -__builtin_inff();
     // the oldest key this lane's query sees: the window's and the block's edges, whichever is later
-    int key_lo = a.window > 0 ? qpos - a.window + 1 : 0;
-    if (a.block > 0) key_lo = max(key_lo, qpos / a.block * a.block);
+    // (keys before the window's edge stay visible when they are among the sequence's kept first ones; the block's edge hides all)
+    const int key_lo = a.window > 0 ? qpos - a.window + 1 : 0;
+    const int blk_lo = a.block > 0 ? qpos / a.block * a.block : 0;
+    const int kept = a.window > 0 ? a.keep_first : 0;
 
     float m = NEG, l = 0.0f;
     f4 o[VB];
@@ -147,6 +149,13 @@ __global__ __launch_bounds__(64 * AW) void attn_softmax_kernel(pcb_attn_softmax_
     int kb_lo = a.window > 0 ? (pos0 - a.window + 1 > 0 ? (pos0 - a.window + 1) / 32 : 0) : 0;
     if (a.block > 0) kb_lo = max(kb_lo, pos0 / a.block * a.block / 32);      // (the tile's first query has the oldest block)
     int kb_hi = last / 32;
+    // kept first keys: the blocks that hold them and lie before the window's first block are walked too.  The walk runs over
+    // indices v in [kb_lo - n_first, kb_hi]: v >= kb_win stands for key block v itself, v < kb_win for block v - (kb_win - n_first).
+    const int kb_win = kb_lo;
+    const int n_first = (a.keep_first > 0 && a.window > 0) ? (kb_win < (a.keep_first + 31) / 32 ? kb_win : (a.keep_first + 31) / 32) : 0;
+    const int v_shift = kb_win - n_first;
+    kb_lo -= n_first;
+    auto block_of = [&](int v) { return v < kb_win ? v - v_shift : v; };
     if (a.n_splits > 1) {                                   // this workgroup's run of the key blocks (it may be empty)
         const int per = (kb_hi - kb_lo + a.n_splits) / a.n_splits;
         kb_lo += (int)blockIdx.z * per;
@@ -156,7 +165,8 @@ __global__ __launch_bounds__(64 * AW) void attn_softmax_kernel(pcb_attn_softmax_
     // the block in work
     constexpr bool PREK = sizeof(E) == 2 ? KSQ <= 4 : KSQ <= 2;
     Frag<E> kn[PREK ? 2 : 1][PREK ? KSQ : 1];
-    auto fetch_k = [&](int kb) {
+    auto fetch_k = [&](int kv) {
+        const int kb = block_of(kv);
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt) {
             int j = kb * 32 + kt * 16 + c;                  // this lane's key row of the K operand
@@ -167,7 +177,8 @@ __global__ __launch_bounds__(64 * AW) void attn_softmax_kernel(pcb_attn_softmax_
         }
     };
     if (PREK && kb_lo + wave <= kb_hi) fetch_k(kb_lo + wave);
-    for (int kb = kb_lo + wave; kb <= kb_hi; kb += AW) {
+    for (int kv = kb_lo + wave; kv <= kb_hi; kv += AW) {
+        const int kb = block_of(kv);
         float s[8];
         Frag<E> kc[PREK ? 2 : 1][PREK ? KSQ : 1];
         if (PREK) {
@@ -175,7 +186,7 @@ __global__ __launch_bounds__(64 * AW) void attn_softmax_kernel(pcb_attn_softmax_
             for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
                 for (int ks = 0; ks < KSQ; ++ks) kc[PREK ? kt : 0][PREK ? ks : 0] = kn[PREK ? kt : 0][PREK ? ks : 0];
-            if (kb + AW <= kb_hi) fetch_k(kb + AW);
+            if (kv + AW <= kb_hi) fetch_k(kv + AW);
         }
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt) {
@@ -189,7 +200,7 @@ __global__ __launch_bounds__(64 * AW) void attn_softmax_kernel(pcb_attn_softmax_
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int key = kb * 32 + kt * 16 + 4 * g + r;
-                const bool seen = key <= qpos && key >= key_lo;
+                const bool seen = key <= qpos && key >= blk_lo && (key >= key_lo || key < kept);
                 s[kt * 4 + r] = seen ? acc[r] * sc : NEG;
             }
         }

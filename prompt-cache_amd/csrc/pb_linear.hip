@@ -53,6 +53,8 @@ __device__ __forceinline__ float apply_act(int act, float v, float param) {
         case PCB_ACT_SOFTCAP: return param * tanhf(v / param);
         case PCB_ACT_RELU: return v > 0.0f ? v : 0.0f;
         case PCB_ACT_GELU_TANH: return 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
+        case PCB_ACT_LOGSIGMOID: return param * (fminf(v, 0.0f) - log1pf(expf(-fabsf(v))));
+        case PCB_ACT_SCALE: return param * v;
         default: return v;
     }
 }
@@ -369,7 +371,7 @@ PCB_EXPORT int pcb_linear(const pcb_linear_args* a, void* stream) {
     PCB_REQUIRE(a->dtype == PCB_BF16 || a->dtype == PCB_F32, PCB_ERR_ARG, "pcb_linear: unknown dtype");
     PCB_REQUIRE(a->M >= 0 && a->N > 0 && a->K > 0 && a->ldx >= a->K && a->ldw >= a->K, PCB_ERR_ARG, "pcb_linear: bad sizes");
     PCB_REQUIRE(a->epilogue >= PCB_EPI_STORE && a->epilogue <= PCB_EPI_SCALE_ADD, PCB_ERR_ARG, "pcb_linear: unknown epilogue");
-    PCB_REQUIRE(a->act >= PCB_ACT_NONE && a->act <= PCB_ACT_GELU_TANH && a->act2 >= PCB_ACT_NONE && a->act2 <= PCB_ACT_GELU_TANH &&
+    PCB_REQUIRE(a->act >= PCB_ACT_NONE && a->act <= PCB_ACT_SCALE && a->act2 >= PCB_ACT_NONE && a->act2 <= PCB_ACT_SCALE &&
                     a->act_split >= 0 &&
                     ((a->act | a->act2) == 0 || a->epilogue == PCB_EPI_STORE ||
                      (a->epilogue == PCB_EPI_SILU_MUL && a->act2 == 0 &&

@@ -388,28 +388,37 @@ __global__ __launch_bounds__(256) void gated_norm_kernel(const float* __restrict
     }
 }
 
-// the same with a norm per run of `group` columns (a head): one wave per (row, group) pair, four pairs per workgroup
+// the same with a norm per run of `group` columns (a head): one wave per (row, group) pair, four pairs per workgroup.  A skip path
+// (x + skip_w[c / skip_group] * skip) and a gate that comes before the norm are this kernel's alone.
 template <typename E>
 __global__ __launch_bounds__(256) void gated_group_norm_kernel(const float* __restrict__ x, int64_t ldx, const float* __restrict__ gain,
                                                                const E* __restrict__ gate, int64_t ldg, E* __restrict__ out, int64_t ldo,
-                                                               float eps, int cols, int group, int64_t n_pairs) {
+                                                               float eps, int cols, int group, int64_t n_pairs, int gate_first,
+                                                               const E* __restrict__ skip, int64_t lds, const float* __restrict__ skip_w,
+                                                               int skip_group) {
     const int lane = threadIdx.x & 63;
     const int64_t pair = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (pair >= n_pairs) return;
     const int per = cols / group;
     const int64_t r = pair / per;
     const int c0 = (int)(pair % per) * group;
+    auto value = [&](int c) {                              // what is normed: x (+ the skip path) (* the gate, when it comes first)
+        float v = x[r * ldx + c];
+        if (skip) v += skip_w[c / skip_group] * to_f32(skip[r * lds + c]);
+        if (gate_first && gate) v *= to_f32(gate[r * ldg + c]);
+        return v;
+    };
     float ss = 0.0f;
     for (int c = lane; c < group; c += 64) {
-        const float v = x[r * ldx + c0 + c];
+        const float v = value(c0 + c);
         ss += v * v;
     }
     ss = wave_sum(ss);
     const float inv = 1.0f / sqrtf(ss / (float)group + eps);
     for (int c = lane; c < group; c += 64) {
-        float v = x[r * ldx + c0 + c] * inv;
+        float v = value(c0 + c) * inv;
         if (gain) v *= gain[c0 + c];
-        if (gate) v *= to_f32(gate[r * ldg + c0 + c]);
+        if (gate && !gate_first) v *= to_f32(gate[r * ldg + c0 + c]);
         out[r * ldo + c0 + c] = from_f32<E>(v);
     }
 }
@@ -437,8 +446,9 @@ __global__ __launch_bounds__(1024) void post_norm_kernel(pcb_post_norm_args a) {
             inv = 1.0f / sqrtf(ss[0] / (float)W + a.eps);
         }
         ss[0] = 0.0f;
+        const float ys = a.y_scale;
         for (int c = threadIdx.x; c < W; c += blockDim.x) {          // (a thread meets its own columns again: no barrier needed)
-            const float v = x[c] + (a.post_gain ? row[c] * inv * a.post_gain[c] : row[c]);
+            const float v = x[c] + ys * (a.post_gain ? row[c] * inv * a.post_gain[c] : row[c]);
             row[c] = v;
             if (!a.rows) x[c] = v;
             ss[0] += v * v;
@@ -453,9 +463,26 @@ __global__ __launch_bounds__(1024) void post_norm_kernel(pcb_post_norm_args a) {
     if (a.x_out)
         for (int c = threadIdx.x; c < W; c += blockDim.x) a.x_out[(int64_t)r * W + c] = row[c];
     if (!a.out) return;
+    E* o = (E*)a.out + (int64_t)r * W;
+    if (a.layer_norm) {
+        // mean first, then the mean of the squared deviations (the row waits in LDS; a thread meets its own columns again)
+        float sm[1] = {0.0f};
+        for (int c = threadIdx.x; c < W; c += blockDim.x) sm[0] += row[c];
+        block_sum<1>(sm, red);
+        const float mean = sm[0] / (float)W;
+        float sv[1] = {0.0f};
+        for (int c = threadIdx.x; c < W; c += blockDim.x) {
+            const float d = row[c] - mean;
+            sv[0] += d * d;
+        }
+        block_sum<1>(sv, red);
+        const float inv = 1.0f / sqrtf(sv[0] / (float)W + a.eps);
+        for (int c = threadIdx.x; c < W; c += blockDim.x)
+            o[c] = from_f32<E>((row[c] - mean) * inv * a.gain[c] + (a.bias ? a.bias[c] : 0.0f));
+        return;
+    }
     block_sum<1>(ss, red);
     const float inv = 1.0f / sqrtf(ss[0] / (float)W + a.eps);
-    E* o = (E*)a.out + (int64_t)r * W;
     for (int c = threadIdx.x; c < W; c += blockDim.x) o[c] = from_f32<E>(row[c] * inv * a.gain[c]);
 }
 
@@ -602,21 +629,25 @@ PCB_EXPORT int pcb_hyper_norm(const pcb_hyper_norm_args* a, void* stream) {
 }
 
 PCB_EXPORT int pcb_gated_norm(const float* x, int64_t ldx, const float* gain, const void* gate, int64_t ldg, void* out, int64_t ldo,
-                              int32_t dtype, float eps, int32_t n_rows, int32_t cols, int32_t group_cols, void* stream) {
+                              int32_t dtype, float eps, int32_t n_rows, int32_t cols, int32_t group_cols, int32_t gate_first,
+                              const void* skip, int64_t lds, const float* skip_w, int32_t skip_group, void* stream) {
     PCB_REQUIRE(PCB_DTYPE_OK(dtype) && n_rows >= 0 && cols > 0 && ldx >= cols && ldo >= cols && (!gate || ldg >= cols), PCB_ERR_ARG,
                 "pcb_gated_norm: bad sizes");
     PCB_REQUIRE(group_cols <= 0 || cols % group_cols == 0, PCB_ERR_ARG, "pcb_gated_norm: the groups must divide the columns");
+    PCB_REQUIRE(!skip || (skip_w && lds >= cols && skip_group > 0 && cols % skip_group == 0), PCB_ERR_ARG,
+                "pcb_gated_norm: a skip path needs its weights and a group size that divides the columns");
     if (n_rows == 0) return PCB_OK;
     PCB_REQUIRE(x && out, PCB_ERR_ARG, "pcb_gated_norm: null pointer");
-    if (group_cols > 0 && group_cols < cols) {
+    if (gate_first || skip) group_cols = group_cols > 0 ? group_cols : cols;       // (the per-group kernel knows these two)
+    if ((group_cols > 0 && group_cols < cols) || gate_first || skip) {
         const int64_t pairs = (int64_t)n_rows * (cols / group_cols);
         const dim3 grid((unsigned)((pairs + 3) / 4));
         if (dtype == PCB_BF16)
             hipLaunchKernelGGL(gated_group_norm_kernel<bf16_t>, grid, dim3(256), 0, (hipStream_t)stream, x, ldx, gain, (const bf16_t*)gate,
-                               ldg, (bf16_t*)out, ldo, eps, cols, group_cols, pairs);
+                               ldg, (bf16_t*)out, ldo, eps, cols, group_cols, pairs, gate_first, (const bf16_t*)skip, lds, skip_w, skip_group);
         else
             hipLaunchKernelGGL(gated_group_norm_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, x, ldx, gain, (const float*)gate,
-                               ldg, (float*)out, ldo, eps, cols, group_cols, pairs);
+                               ldg, (float*)out, ldo, eps, cols, group_cols, pairs, gate_first, (const float*)skip, lds, skip_w, skip_group);
         return pcb_check_launch("gated_group_norm_kernel");
     }
     if (dtype == PCB_BF16)

@@ -16,10 +16,10 @@ _lib: Optional[C.CDLL] = None
 
 BF16, F32 = 0, 1
 EPI_STORE, EPI_SILU_MUL, EPI_SCALE_ADD = 0, 1, 2
-ACT_NONE, ACT_SILU, ACT_SIGMOID, ACT_RELU2, ACT_SOFTPLUS, ACT_SOFTCAP, ACT_RELU, ACT_GELU_TANH = 0, 1, 2, 3, 4, 5, 6, 7
+ACT_NONE, ACT_SILU, ACT_SIGMOID, ACT_RELU2, ACT_SOFTPLUS, ACT_SOFTCAP, ACT_RELU, ACT_GELU_TANH, ACT_LOGSIGMOID, ACT_SCALE = range(10)
 NORM_NONE, NORM_RMS, NORM_DYT = 0, 1, 2
 SCORE_SIGMOID, SCORE_SOFTMAX = 0, 1
-ABI_VERSION = 3
+ABI_VERSION = 4
 DTYPES = {torch.bfloat16: BF16, torch.float32: F32}
 
 
@@ -73,7 +73,7 @@ class AttnSoftmaxArgs(C.Structure):
                 ("v_slot_stride", _i64), ("v_head_stride", _i64), ("v_stride", _i64), ("v_cols", _i32),
                 ("H", _i32), ("Hkv", _i32), ("dim", _i32), ("vdim", _i32), ("scale", _f32), ("window", _i32),
                 ("gate", _vp), ("ldg", _i64), ("out", _vp), ("ldo", _i64), ("n_splits", _i32), ("part", _vp),
-                ("block", _i32), ("sink", _vp), ("gate_per_head", _i32), ("head_rows", _i32)]
+                ("block", _i32), ("sink", _vp), ("gate_per_head", _i32), ("head_rows", _i32), ("keep_first", _i32)]
 
 
 class DecayAttnArgs(C.Structure):
@@ -96,7 +96,8 @@ class PostNormArgs(C.Structure):
     """``pcb_post_norm_args`` (field for field)."""
     _fields_ = [("struct_bytes", C.c_uint32), ("dtype", _i32),
                 ("x", _vp), ("y", _vp), ("gate", _vp), ("ldg", _i64), ("post_gain", _vp), ("gain", _vp),
-                ("out", _vp), ("x_out", _vp), ("rows", _vp), ("eps", _f32), ("n_rows", _i32), ("width", _i32)]
+                ("out", _vp), ("x_out", _vp), ("rows", _vp), ("eps", _f32), ("n_rows", _i32), ("width", _i32),
+                ("y_scale", _f32), ("layer_norm", _i32), ("bias", _vp)]
 
 
 class HeadPrepSeg(C.Structure):
@@ -123,6 +124,15 @@ class MlstmArgs(C.Structure):
                 ("from_nothing", _i32), ("log_f_sum", _vp), ("end_slots", _vp), ("end_state", _vp), ("end_slot_stride", _i64)]
 
 
+class GlaArgs(C.Structure):
+    """``pcb_gla_args`` (field for field)."""
+    _fields_ = [("struct_bytes", C.c_uint32), ("dtype", _i32),
+                ("q", _vp), ("k", _vp), ("v", _vp), ("ldq", _i64), ("ldk", _i64), ("ldv", _i64),
+                ("ld", _vp), ("ldld", _i64), ("dcols", _i32), ("ld_coef", _vp), ("v_scale", _vp), ("ldvs", _i64),
+                ("reqs", _vp), ("n_reqs", _i32), ("state", _vp), ("slot_stride", _i64),
+                ("H", _i32), ("Hk", _i32), ("dim", _i32), ("vdim", _i32), ("q_scale", _f32), ("out", _vp), ("ldo", _i64), ("ld_sum", _vp)]
+
+
 # name -> (restype, argtypes); mirrors include/promptcache_blocks.h one to one
 SIGNATURES = {
     "pcb_version": (C.c_int, []),
@@ -139,7 +149,7 @@ SIGNATURES = {
     "pcb_attn_talk": (C.c_int, [C.POINTER(AttnTalkArgs), _vp]),
     "pcb_embed_pos_rows": (C.c_int, [_vp, _vp, _i32, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _i32, _vp]),
     "pcb_hyper_norm": (C.c_int, [C.POINTER(HyperNormArgs), _vp]),
-    "pcb_gated_norm": (C.c_int, [_vp, _i64, _vp, _vp, _i64, _vp, _i64, _i32, _f32, _i32, _i32, _i32, _vp]),
+    "pcb_gated_norm": (C.c_int, [_vp, _i64, _vp, _vp, _i64, _vp, _i64, _i32, _f32, _i32, _i32, _i32, _i32, _vp, _i64, _vp, _i32, _vp]),
     "pcb_router_select": (C.c_int, [_vp, _i32, _i32, _i32, _i32, _vp, _i32, _i32, _i32, _vp, _vp, _vp]),
     "pcb_moe_mix": (C.c_int, [_vp, _vp, _vp, _vp, _i32, _i32, _vp, _i32, _i32, _i32, _vp]),
     "pcb_attn_softmax": (C.c_int, [C.POINTER(AttnSoftmaxArgs), _vp]),
@@ -152,6 +162,7 @@ SIGNATURES = {
     "pcb_head_prep": (C.c_int, [C.POINTER(HeadPrepArgs), _vp]),
     "pcb_mlstm": (C.c_int, [C.POINTER(MlstmArgs), _vp]),
     "pcb_mlstm_chain": (C.c_int, [_vp, _vp, _vp, _vp, _i64, _vp, _i32, _i32, _i32, _i32, _vp]),
+    "pcb_gla": (C.c_int, [C.POINTER(GlaArgs), _vp]),
 }
 
 
@@ -403,18 +414,24 @@ def hyper_norm(streams: torch.Tensor, *, y=None, mix=None, out_w=None, in_w=None
 
 
 def gated_norm(x: torch.Tensor, gain: Optional[torch.Tensor], gate: Optional[torch.Tensor], ldg: int, out: torch.Tensor, eps: float,
-               n_rows: int, group: int = 0) -> None:
+               n_rows: int, group: int = 0, gate_first: bool = False, skip: Optional[torch.Tensor] = None, lds: int = 0,
+               skip_w: Optional[torch.Tensor] = None, skip_group: int = 0) -> None:
     """``x`` fp32 [rows, cols]; ``gate`` E, a column block (row stride ``ldg``) of a wider matrix; ``out`` E [rows, cols].
-    ``group`` > 0: a norm per run of that many columns (per head) instead of one over the row."""
-    _want(x, torch.float32, "gated_norm x"); _want(gain, torch.float32, "gated_norm gain")
+    ``group`` > 0: a norm per run of that many columns (per head) instead of one over the row.  ``skip`` (E rows of stride
+    ``lds``) with ``skip_w`` (fp32, one weight per ``skip_group`` columns): x + skip_w * skip stands for x.  ``gate_first``: the
+    gate is applied before the norm."""
+    _want(x, torch.float32, "gated_norm x"); _want(gain, torch.float32, "gated_norm gain"); _want(skip_w, torch.float32, "gated_norm skip_w")
     cols = x.shape[-1]
     assert out.is_contiguous() and out.shape[-1] == cols and x.shape[0] >= n_rows and out.shape[0] >= n_rows
     assert gain is None or gain.numel() == cols
     if gate is not None:
         assert gate.dtype == out.dtype and gate.is_cuda and ldg >= cols
+    if skip is not None:
+        assert skip.dtype == out.dtype and skip.is_cuda and lds >= cols and skip_group > 0 and cols % skip_group == 0
+        assert skip_w is not None and skip_w.numel() == cols // skip_group
     assert group == 0 or cols % group == 0
     check(load().pcb_gated_norm(_p(x), cols, _p(gain), _p(gate), ldg, _p(out), cols, _code(out), float(eps), n_rows, cols, int(group),
-                                _stream()), "pcb_gated_norm")
+                                int(gate_first), _p(skip), int(lds), _p(skip_w), int(skip_group), _stream()), "pcb_gated_norm")
 
 
 def router_select(logits: torch.Tensor, top: int, expert: torch.Tensor, weight: torch.Tensor, n_rows: int, *, score_fn: int,
@@ -442,7 +459,7 @@ def attn_softmax(q: torch.Tensor, ldq: int, tiles: torch.Tensor, n_tiles: int, k
                  v_offset: int, v_strides, v_cols: bool, H: int, Hkv: int, dim: int, vdim: int, scale: float, out: torch.Tensor, *,
                  q_scale: Optional[torch.Tensor] = None, window: int = 0, gate: Optional[torch.Tensor] = None, ldg: int = 0,
                  n_splits: int = 1, part: Optional[torch.Tensor] = None, block: int = 0, sink: Optional[torch.Tensor] = None,
-                 gate_per_head: bool = False, head_rows: bool = False) -> None:
+                 gate_per_head: bool = False, head_rows: bool = False, keep_first: int = 0) -> None:
     """``q``: E rows (row stride ``ldq``, head h at column h * dim); ``kcache`` with ``k_strides`` = (slot, head, row) strides in
     elements; the values start ``v_offset`` elements into ``vcache`` (which may be the same plane) with ``v_strides`` = (slot, head,
     row) strides, or (slot, head, column) strides when ``v_cols`` (a cache kept column by column, columns readable in multiples of
@@ -450,7 +467,8 @@ def attn_softmax(q: torch.Tensor, ldq: int, tiles: torch.Tensor, n_tiles: int, k
     workgroups over runs of the keys, merged by a second launch; ``part``: fp32 scratch of ``attn_softmax_part(rows, H, n_splits,
     vdim)`` floats.  ``block`` > 0: a key is seen only inside the query's own block of that many positions; ``sink`` fp32 [H]: one
     more exp(sink[h]) in the denominator; ``gate_per_head``: the gate has one column per head; ``head_rows``: every tile has one row and
-    there is one key head -- a workgroup then serves 16 heads of the row at once."""
+    there is one key head -- a workgroup then serves 16 heads of the row at once; ``keep_first`` > 0: behind a window the keys at
+    positions below it stay visible."""
     _want(tiles, torch.int32, "attn_softmax tiles"); _want(q_scale, torch.float32, "attn_softmax q_scale")
     _want(sink, torch.float32, "attn_softmax sink")
     assert sink is None or sink.numel() == H
@@ -461,7 +479,7 @@ def attn_softmax(q: torch.Tensor, ldq: int, tiles: torch.Tensor, n_tiles: int, k
     a = AttnSoftmaxArgs(C.sizeof(AttnSoftmaxArgs), _code(q), _p(q), ldq, _p(q_scale), _p(tiles), n_tiles, _p(kcache),
                         vcache.data_ptr() + v_offset * es, int(k_strides[0]), int(k_strides[1]), int(k_strides[2]), int(v_strides[0]),
                         int(v_strides[1]), int(v_strides[2]), int(v_cols), H, Hkv, dim, vdim, float(scale), int(window), _p(gate), ldg,
-                        _p(out), out.shape[-1], int(n_splits), _p(part), int(block), _p(sink), int(gate_per_head), int(head_rows))
+                        _p(out), out.shape[-1], int(n_splits), _p(part), int(block), _p(sink), int(gate_per_head), int(head_rows), int(keep_first))
     if n_splits > 1:
         _want(part, torch.float32, "attn_softmax part")
         assert part.numel() >= attn_softmax_part(out.shape[0], H, n_splits, vdim)
@@ -542,11 +560,13 @@ def state_chain(local: torch.Tensor, start: torch.Tensor, state: torch.Tensor, c
 
 # ---- sublayers between two norms, per-head preparation, matrix memories ----------------------------------------------------------
 def post_norm(x: torch.Tensor, *, y=None, gate=None, ldg: int = 0, post_gain=None, gain=None, out=None, x_out=None, rows=None,
-              eps: float = 1e-6, n_rows: Optional[int] = None) -> None:
+              eps: float = 1e-6, n_rows: Optional[int] = None, y_scale: float = 1.0, layer_norm: bool = False, bias=None) -> None:
     """``x`` fp32 [T, W] (the residual).  With ``y`` (fp32 [T, W]): x += norm(y * gate) * post_gain (``gate`` E rows of stride
     ``ldg``; without ``post_gain`` the gated y is added as it is).  With ``out`` (E): out = norm(x) * gain, for the rows ``rows``
-    only if given (then x itself is not rewritten); ``x_out`` fp32 receives those rows of x."""
-    _want(x, torch.float32, "post_norm x")
+    only if given (then x itself is not rewritten); ``x_out`` fp32 receives those rows of x.  ``y_scale``: the factor on what is
+    added to x; ``layer_norm``: out = (x - mean) / sqrt(variance + eps) * gain + bias instead of the RMS form."""
+    _want(x, torch.float32, "post_norm x"); _want(bias, torch.float32, "post_norm bias")
+    assert bias is None or (layer_norm and bias.numel() == x.shape[-1])
     T, W = x.shape
     n = (rows.numel() if rows is not None else T) if n_rows is None else n_rows
     for t, nm in ((y, "y"), (post_gain, "post_gain"), (gain, "gain"), (x_out, "x_out")):
@@ -566,7 +586,7 @@ def post_norm(x: torch.Tensor, *, y=None, gate=None, ldg: int = 0, post_gain=Non
     if rows is not None:
         _want(rows, torch.int32, "post_norm rows")
     a = PostNormArgs(C.sizeof(PostNormArgs), code, _p(x), _p(y), _p(gate), ldg, _p(post_gain), _p(gain), _p(out), _p(x_out), _p(rows),
-                     float(eps), n, W)
+                     float(eps), n, W, float(y_scale), int(layer_norm), _p(bias))
     check(load().pcb_post_norm(C.byref(a), _stream()), "pcb_post_norm")
 
 
@@ -642,3 +662,27 @@ def mlstm_chain(local: torch.Tensor, log_f_sum: torch.Tensor, start: torch.Tenso
     assert log_f_sum.numel() >= local.shape[0] * H and chains.numel() >= 4 * n_chains
     check(load().pcb_mlstm_chain(_p(local), _p(log_f_sum), _p(start), _p(state), rec, _p(chains), n_chains, H, dim, vdim, _stream()),
           "pcb_mlstm_chain")
+
+
+def gla(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, ld: torch.Tensor, lds_: tuple, dcols: int, reqs: torch.Tensor, n_reqs: int,
+        state: torch.Tensor, H: int, Hk: int, dim: int, vdim: int, q_scale: float, out: Optional[torch.Tensor], *,
+        ld_coef: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None, ldvs: int = 0,
+        ld_sum: Optional[torch.Tensor] = None) -> None:
+    """Linear attention with a decay per token: ``q``, ``k`` (``Hk`` heads), ``v`` (``H`` heads) E rows with row strides
+    ``lds_`` = (ldq, ldk, ldv, ldld); ``ld`` fp32 rows of log decays, ``dcols`` = ``dim`` (one per key channel) or 1 (one per head),
+    times ``ld_coef`` [H] when given; ``v_scale`` fp32 rows (stride ``ldvs``) of one step size per head; ``state`` fp32
+    [slots, H, dim, vdim]; ``out`` fp32 [rows, H * vdim] or None (states only; ``ld_sum`` fp32 [n_reqs, H * dcols] then receives
+    the sums of the log decays)."""
+    _want(reqs, torch.int32, "gla reqs"); _want(state, torch.float32, "gla state"); _want(out, torch.float32, "gla out")
+    _want(ld_coef, torch.float32, "gla ld_coef"); _want(ld_sum, torch.float32, "gla ld_sum")
+    assert q.dtype == k.dtype == v.dtype and q.is_cuda and ld.dtype == torch.float32 and ld.is_cuda
+    assert reqs.numel() >= 4 * n_reqs and state.shape[-3:] == (H, dim, vdim) and dcols in (1, dim)
+    assert out is None or out.shape[-1] == H * vdim
+    assert v_scale is None or (v_scale.dtype == torch.float32 and ldvs >= H)
+    assert ld_coef is None or ld_coef.numel() == H
+    assert ld_sum is None or ld_sum.numel() >= n_reqs * H * dcols
+    ldq, ldk, ldv, ldld = (int(x) for x in lds_)
+    a = GlaArgs(C.sizeof(GlaArgs), _code(q), _p(q), _p(k), _p(v), ldq, ldk, ldv, _p(ld), ldld, int(dcols), _p(ld_coef), _p(v_scale),
+                int(ldvs), _p(reqs), n_reqs, _p(state), H * dim * vdim, H, Hk, dim, vdim, float(q_scale), _p(out),
+                H * vdim if out is not None else 0, _p(ld_sum))
+    check(load().pcb_gla(C.byref(a), _stream()), "pcb_gla")

@@ -22,7 +22,7 @@ from typing import Callable, List, Optional, Tuple
 import torch
 
 from ..pml import Preprocessor, PreprocessorList, escape_xml  # noqa: F401  (re-exported like the reference)
-from .config import (FALCON_SHAPES, MPT_SHAPES, SHAPES, DibizenShape, FalconShape, FivesunShape, KazolornShape, LlamaShape, MptShape,
+from .config import (FALCON_SHAPES, MPT_SHAPES, SHAPES, BepepelShape, DibizenShape, FalconShape, FivesunShape, KazolornShape, LlamaShape, MptShape,
                      architecture_of)
 from .tokenizer import StandInTokenizer
 
@@ -404,7 +404,48 @@ class Fivesun(LanguageModel):
         return [t % self.config.vocab_size for t in super().encode(text)]
 
 
-ADAPTERS = {"llama": Llama2, "falcon": Falcon, "mpt": Mpt, "kazolorn": Kazolorn, "dibizen": Dibizen, "fivesun": Fivesun}
+class Bepepel(LanguageModel):
+    """Adapter of the Bepepel design (``config.BepepelShape``, ``bepepel_hip.BepepelHIP``).  A checkpoint directory holds
+    ``config.json`` and ``model.safetensors``; without one, ``shape=`` plus ``random_init=True`` (or ``weights=``) gives seeded
+    random weights.  ``dtype``: ``torch.bfloat16`` (serving) or ``torch.float32`` (everything in true 32-bit)."""
+
+    def __init__(self, name: Optional[str] = None, device: str = "cuda:0", shape: Optional[BepepelShape] = None,
+                 weights=None, tokenizer=None, random_init: bool = False, seed: int = 0, dtype=torch.bfloat16, **_kwargs):
+        from .bepepel_hip import BepepelHIP
+        from . import weights as W
+
+        if weights is not None:
+            assert shape is not None, "pass shape= together with weights="
+        elif name is not None and os.path.isdir(name):
+            shape = shape or BepepelShape.from_dir(name)
+            weights = W.load_bepepel_safetensors(name, shape)
+        else:
+            if shape is None or not random_init:
+                raise FileNotFoundError(f"no checkpoint directory {name!r}: pass one, or shape= with random_init=True")
+            weights = W.make_bepepel_weights(shape, seed, device=device)
+        if tokenizer is None:
+            tokenizer = StandInTokenizer(max(shape.vocab_size, 512))
+        model = BepepelHIP(shape, weights, device=device, dtype=dtype)
+        self.formatter = FormatConversation(system=("", "\n\n", ""), user=("User: ", "\n\nAssistant:"), assistant=(" ", "\n\n"))
+        super().__init__(name or shape.name, model, tokenizer, [tokenizer.eos_token_id], [])
+
+    def get_formatter(self) -> Callable[[str], str]:
+        return self.formatter
+
+    def get_cache_shape(self) -> Tuple[int, int, int]:
+        """(layers, kv heads, key size) of the first layer that keeps rows per token (zeros when none does); every layer also
+        keeps states of its own shapes (``BepepelHIP.new_arena`` knows them all)."""
+        for l in self.config.layers:
+            if l.kind == "parallel":
+                return len(self.config.layers), l.left.kv_heads, l.left.dim
+        return len(self.config.layers), 0, 0
+
+    def encode(self, text: str) -> List[int]:
+        return [t % self.config.vocab_size for t in super().encode(text)]
+
+
+ADAPTERS = {"llama": Llama2, "falcon": Falcon, "mpt": Mpt, "kazolorn": Kazolorn, "dibizen": Dibizen, "fivesun": Fivesun,
+            "bepepel": Bepepel}
 
 
 def load_language_model(path: str, **kwargs) -> LanguageModel:

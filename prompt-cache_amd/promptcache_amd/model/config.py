@@ -8,6 +8,7 @@ from __future__ import annotations
 import json
 import os
 from dataclasses import dataclass, asdict
+from typing import Optional
 
 
 @dataclass
@@ -629,6 +630,230 @@ class FivesunShape:
             layers.append(lay)
         return cls(vocab_size=vocab, hidden_size=width, norm_eps=1e-6, layers=layers, embed_scale=width ** 0.5, name=name)
 
+@dataclass
+class BepepelAttention:
+    """The softmax half of a Bepepel ``parallel`` mixer: ``heads`` query heads over ``kv_heads`` key/value heads (``dim`` query/key
+    and ``vdim`` value columns), projections with biases, a causal convolution of ``conv`` taps per channel on q, k and v (0: none),
+    interleaved rotary pairs on the first ``rot_dims`` columns (``rot_scaling``: None, or (factor, low, high, original) of the
+    wavelength-dependent frequency scaling), unit-RMS queries and keys, score = ``scale`` q.k, a sliding window of ``window``
+    positions (0: all earlier keys) that also keeps the sequence's first ``keep_first`` positions visible."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    conv: int = 0
+    window: int = 0
+    keep_first: int = 0
+    rot_base: float = 10000.0
+    rot_dims: int = 0
+    rot_scaling: Optional[tuple] = None
+
+
+@dataclass
+class BepepelSSD:
+    """The state-space half of a Bepepel ``parallel`` mixer (Mamba-2): ``heads`` heads of ``vdim`` channels, a ``state`` x ``vdim``
+    matrix state per head with one scalar decay per head and token, B and C shared by the heads of each of ``groups`` groups, a
+    causal convolution of ``conv`` taps over x | B | C (0: none), the gated output normed in ``norm_groups`` equal parts."""
+    heads: int
+    vdim: int
+    state: int
+    groups: int = 1
+    norm_groups: int = 1
+    conv: int = 0
+
+    @property
+    def inner(self) -> int:
+        return self.heads * self.vdim
+
+    @property
+    def conv_channels(self) -> int:
+        return self.inner + 2 * self.groups * self.state
+
+    @property
+    def in_columns(self) -> int:
+        return 2 * self.inner + 2 * self.groups * self.state + self.heads
+
+
+@dataclass
+class BepepelLayer:
+    """One layer of a Bepepel stack.  ``kind``: which mixer it has --
+
+    * ``"gla"``: gated linear attention, ``heads`` heads with a ``dim`` x ``vdim`` matrix state each and one decay per key channel
+      and token, sigmoid(low-rank projection)^(1 / ``tau``); per-head unit-RMS outputs with a shared gain, a SiLU output gate;
+    * ``"parallel"``: ``left`` (``BepepelAttention``) and ``right`` (``BepepelSSD``) read the same input and their results are added
+      as ``left_scale`` * left + ``right_scale`` * right.
+
+    ``ff_kind``: "" (no feed-forward), "dense" (a gated unit of width ``ff``, tanh-form GELU) or "moe" (``experts`` gated SiLU units
+    of width ``expert_ff`` of which each token uses the ``top`` with the largest router logits, weighted by the softmax over those
+    logits, plus -- ``shared_ff`` > 0 -- one unit of that width that every token uses)."""
+    kind: str
+    heads: int = 0
+    dim: int = 0
+    vdim: int = 0
+    tau: float = 1.0
+    a_rank: int = 0
+    left: Optional[BepepelAttention] = None
+    right: Optional[BepepelSSD] = None
+    left_scale: float = 1.0
+    right_scale: float = 1.0
+    ff_kind: str = ""
+    ff: int = 0
+    experts: int = 0
+    top: int = 0
+    expert_ff: int = 0
+    shared_ff: int = 0
+
+
+@dataclass
+class BepepelShape:
+    """Bepepel: decoder-only, pre-norm layers (layer norms with weight and bias) whose results enter the residual stream times
+    ``residual_mult``, mixers gated linear attention or a softmax attention and a Mamba-2 side by side, dense or mixture-of-experts
+    feed-forwards, logits times ``logit_scale``.  Every size and constant comes from ``config.json`` (``from_config``); the low rank
+    of the decay projection is a tensor's shape and is filled in by the weight loader (``a_rank`` 0: not known yet)."""
+    vocab_size: int
+    hidden_size: int
+    norm_eps: float
+    layers: list
+    residual_mult: float = 1.0
+    logit_scale: float = 1.0
+    name: str = "bepepel"
+
+    ARCHITECTURE = "Bepepel"
+    KINDS = ("gla", "parallel")
+
+    @property
+    def num_hidden_layers(self) -> int:
+        return len(self.layers)
+
+    @classmethod
+    def from_config(cls, c: dict, name: str = "bepepel") -> "BepepelShape":
+        if c.get("architecture") != cls.ARCHITECTURE:
+            raise ValueError(f"config.json describes {c.get('architecture')!r}, not {cls.ARCHITECTURE}")
+        layers = []
+        for i, lc in enumerate(c["layers"]):
+            kind, m = lc.get("type"), lc.get("mixer") or {}
+            if kind == "gla":
+                dim = int(m["dim"])
+                lay = BepepelLayer(kind, heads=int(m["heads"]), dim=dim, vdim=int(m.get("vdim") or dim), tau=float(m.get("tau", 1.0)),
+                                   a_rank=int(m.get("a_rank") or 0))
+            elif kind == "parallel":
+                a, b = m["left"], m["right"]
+                rot, mask = a.get("rot") or {}, a.get("mask") or {}
+                sc = rot.get("scaling")
+                heads, dim = int(a["heads"]), int(a["dim"])
+                left = BepepelAttention(heads=heads, kv_heads=int(a.get("kv_heads") or heads), dim=dim, vdim=int(a.get("vdim") or dim),
+                                        scale=float(a.get("scale", dim ** -0.5)), conv=int(a.get("conv") or 0),
+                                        window=int(mask.get("size") or 0), keep_first=int(mask.get("keep_first") or 0),
+                                        rot_base=float(rot.get("base", 10000.0)), rot_dims=int(rot.get("dims", dim if rot else 0)),
+                                        rot_scaling=(float(sc["factor"]), float(sc["low"]), float(sc["high"]), float(sc["original"]))
+                                        if sc else None)
+                right = BepepelSSD(heads=int(b["heads"]), vdim=int(b["vdim"]), state=int(b["state"]), groups=int(b.get("groups") or 1),
+                                   norm_groups=int(b.get("norm_groups") or 1), conv=int(b.get("conv") or 0))
+                lay = BepepelLayer(kind, left=left, right=right, left_scale=float(m.get("left_scale", 1.0)),
+                                   right_scale=float(m.get("right_scale", 1.0)))
+            else:
+                raise ValueError(f"layer {i}: unknown mixer type {kind!r}")
+            mlp = lc.get("mlp")
+            if mlp:
+                fk = mlp.get("kind", "dense")
+                if fk == "dense":
+                    lay.ff_kind, lay.ff = "dense", int(mlp["ff"])
+                elif fk == "moe":
+                    lay.ff_kind, lay.experts, lay.top = "moe", int(mlp["router"]["experts"]), int(mlp["router"]["top"])
+                    lay.expert_ff = int(mlp["expert"]["ff"])
+                    lay.shared_ff = int((mlp.get("shared") or {}).get("ff") or 0)
+                else:
+                    raise ValueError(f"layer {i}: unknown feed-forward kind {fk!r}")
+            layers.append(lay)
+        shape = cls(vocab_size=int(c["vocab"]), hidden_size=int(c["width"]), norm_eps=float((c.get("norm") or {}).get("eps", 1e-6)),
+                    layers=layers, residual_mult=float(c.get("residual_mult", 1.0)), logit_scale=float(c.get("logit_scale", 1.0)),
+                    name=name)
+        shape.check()
+        return shape
+
+    def check(self) -> None:
+        for i, l in enumerate(self.layers):
+            if l.kind not in self.KINDS:
+                raise ValueError(f"layer {i}: unknown mixer type {l.kind!r}")
+            if l.kind == "gla":
+                if min(l.heads, l.dim, l.vdim) < 1 or l.tau <= 0:
+                    raise ValueError(f"layer {i}: gated linear attention needs heads, sizes and a positive tau")
+            else:
+                a, b = l.left, l.right
+                if a.heads % a.kv_heads:
+                    raise ValueError(f"layer {i}: {a.heads} query heads do not divide over {a.kv_heads} key heads")
+                if a.rot_dims % 2 or a.rot_dims > a.dim:
+                    raise ValueError(f"layer {i}: {a.rot_dims} rotated columns of {a.dim}")
+                if b.heads % b.groups or (b.heads * b.vdim) % b.norm_groups:
+                    raise ValueError(f"layer {i}: {b.heads} heads over {b.groups} groups, {b.heads * b.vdim} channels in {b.norm_groups} parts")
+            if l.ff_kind == "moe" and not 1 <= l.top <= l.experts:
+                raise ValueError(f"layer {i}: top {l.top} of {l.experts} experts")
+
+    @classmethod
+    def from_dir(cls, path: str) -> "BepepelShape":
+        with open(os.path.join(path, "config.json")) as f:
+            return cls.from_config(json.load(f), name=os.path.basename(os.path.normpath(path)))
+
+    def to_config(self) -> dict:
+        """The ``config.json`` form (what ``from_config`` reads)."""
+        out = []
+        for l in self.layers:
+            if l.kind == "gla":
+                mixer = {"dim": l.dim, "heads": l.heads, "tau": l.tau, "vdim": l.vdim}
+                if l.a_rank:
+                    mixer["a_rank"] = l.a_rank
+            else:
+                a, b = l.left, l.right
+                left = {"dim": a.dim, "heads": a.heads, "kv_heads": a.kv_heads, "scale": a.scale, "vdim": a.vdim}
+                if a.conv:
+                    left["conv"] = a.conv
+                if a.window:
+                    left["mask"] = {"keep_first": a.keep_first, "size": a.window}
+                if a.rot_dims:
+                    left["rot"] = {"base": a.rot_base, "dims": a.rot_dims}
+                    if a.rot_scaling:
+                        left["rot"]["scaling"] = dict(zip(("factor", "low", "high", "original"), a.rot_scaling))
+                right = {"groups": b.groups, "heads": b.heads, "norm_groups": b.norm_groups, "state": b.state, "vdim": b.vdim}
+                if b.conv:
+                    right["conv"] = b.conv
+                mixer = {"left": left, "left_scale": l.left_scale, "right": right, "right_scale": l.right_scale}
+            if l.ff_kind == "dense":
+                mlp = {"ff": l.ff, "kind": "dense"}
+            elif l.ff_kind == "moe":
+                mlp = {"expert": {"ff": l.expert_ff}, "kind": "moe", "router": {"experts": l.experts, "top": l.top}}
+                if l.shared_ff:
+                    mlp["shared"] = {"ff": l.shared_ff}
+            else:
+                mlp = None
+            out.append({"type": l.kind, "mixer": mixer, "mlp": mlp})
+        return {"architecture": self.ARCHITECTURE, "layers": out, "logit_scale": self.logit_scale, "norm": {"eps": self.norm_eps},
+                "residual_mult": self.residual_mult, "vocab": self.vocab_size, "width": self.hidden_size}
+
+    @classmethod
+    def uniform(cls, vocab: int, width: int, pattern, heads: int, kv_heads: int, dim: int, experts: int = 0, top: int = 0,
+                expert_ff: int = 0, dense_ff: int = 0, window: int = 0, keep_first: int = 0, ssd_state: int = 128, ssd_vdim: int = 64,
+                name: str = "bepepel") -> "BepepelShape":
+        """A stack whose layers follow ``pattern`` (a sequence of mixer kinds), all with the same sizes: ``experts`` > 0 gives every
+        layer a mixture-of-experts feed-forward with a shared expert, else ``dense_ff`` > 0 a dense one."""
+        layers = []
+        for kind in pattern:
+            if kind == "gla":
+                lay = BepepelLayer(kind, heads=heads, dim=dim, vdim=dim, tau=8.0, a_rank=16)
+            else:
+                left = BepepelAttention(heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, scale=1.0 / 8.0, conv=3, window=window,
+                                        keep_first=keep_first, rot_base=500000.0, rot_dims=dim // 2,
+                                        rot_scaling=(4.0, 1.0, 4.0, 2048.0))
+                sh = max(width // ssd_vdim, 1)
+                right = BepepelSSD(heads=sh, vdim=ssd_vdim, state=ssd_state, groups=1, norm_groups=1, conv=4)
+                lay = BepepelLayer(kind, left=left, right=right, left_scale=1.0, right_scale=1.0)
+            if experts:
+                lay.ff_kind, lay.experts, lay.top, lay.expert_ff, lay.shared_ff = "moe", experts, top, expert_ff, expert_ff
+            elif dense_ff:
+                lay.ff_kind, lay.ff = "dense", dense_ff
+            layers.append(lay)
+        return cls(vocab_size=vocab, hidden_size=width, norm_eps=1e-6, layers=layers, residual_mult=0.5, logit_scale=1.0, name=name)
+
 
 def architecture_of(path: str) -> str:
     """Which model family a checkpoint directory holds: ``architecture`` (Kazolorn) or HF's ``model_type``."""
@@ -640,4 +865,6 @@ def architecture_of(path: str) -> str:
         return "dibizen"
     if c.get("architecture") == FivesunShape.ARCHITECTURE:
         return "fivesun"
+    if c.get("architecture") == BepepelShape.ARCHITECTURE:
+        return "bepepel"
     return str(c.get("model_type", "llama"))

@@ -520,3 +520,103 @@ def load_fivesun_safetensors(path: str, cfg):
         if tuple(raw[k].shape) != tuple(shp) and raw[k].numel() != 1:
             raise ValueError(f"{path}: {k} has shape {tuple(raw[k].shape)}, the configuration implies {tuple(shp)}")
     return {k: raw[k] for k in want}
+
+
+def bepepel_weight_shapes(cfg) -> Dict[str, tuple]:
+    """Tensor names and shapes of a Bepepel checkpoint (``model.safetensors``): ``embed``; per layer ``l{i}.norm1`` (+ ``.b``), the
+    mixer's ``l{i}.mix.*`` (gla: ``q k v g o norm a1 a2 a2.b``; parallel: ``left.q|k|v`` each with ``.b`` and, with a convolution,
+    ``.conv``, ``left.o``, ``right.in conv conv.b dt_bias A_log D norm o``) and, with a feed-forward, ``l{i}.norm2`` (+ ``.b``) and
+    ``l{i}.mlp.gate|up|down`` (dense) or ``l{i}.mlp.router`` (+ ``.b``), ``l{i}.mlp.e{j}.gate|up|down`` and ``l{i}.mlp.shared.*``;
+    then ``final.norm`` (+ ``.b``) and ``head``."""
+    W = cfg.hidden_size
+    s = {"embed": (cfg.vocab_size, W)}
+
+    def unit(pre, ff):
+        s[pre + "gate"], s[pre + "up"], s[pre + "down"] = (ff, W), (ff, W), (W, ff)
+
+    for i, l in enumerate(cfg.layers):
+        p, m = f"l{i}.", f"l{i}.mix."
+        s[p + "norm1"], s[p + "norm1.b"] = (W,), (W,)
+        if l.kind == "gla":
+            HD, HV = l.heads * l.dim, l.heads * l.vdim
+            s[m + "q"], s[m + "k"], s[m + "v"], s[m + "g"], s[m + "o"], s[m + "norm"] = (HD, W), (HD, W), (HV, W), (HV, W), (W, HV), (l.vdim,)
+            s[m + "a1"], s[m + "a2"], s[m + "a2.b"] = (l.a_rank, W), (HD, l.a_rank), (HD,)
+        else:
+            a, b = l.left, l.right
+            for nm, n in (("q", a.heads * a.dim), ("k", a.kv_heads * a.dim), ("v", a.kv_heads * a.vdim)):
+                s[m + "left." + nm], s[m + "left." + nm + ".b"] = (n, W), (n,)
+                if a.conv:
+                    s[m + "left." + nm + ".conv"] = (n, a.conv)
+            s[m + "left.o"] = (W, a.heads * a.vdim)
+            r = m + "right."
+            s[r + "in"] = (b.in_columns, W)
+            if b.conv:
+                s[r + "conv"], s[r + "conv.b"] = (b.conv_channels, b.conv), (b.conv_channels,)
+            s[r + "dt_bias"], s[r + "A_log"], s[r + "D"], s[r + "norm"], s[r + "o"] = (b.heads,), (b.heads,), (b.heads,), (b.inner,), (W, b.inner)
+        if l.ff_kind:
+            s[p + "norm2"], s[p + "norm2.b"] = (W,), (W,)
+            if l.ff_kind == "dense":
+                unit(p + "mlp.", l.ff)
+            else:
+                s[p + "mlp.router"], s[p + "mlp.router.b"] = (l.experts, W), (l.experts,)
+                for j in range(l.experts):
+                    unit(p + f"mlp.e{j}.", l.expert_ff)
+                if l.shared_ff:
+                    unit(p + "mlp.shared.", l.shared_ff)
+    s["final.norm"], s["final.norm.b"], s["head"] = (W,), (W,), (cfg.vocab_size, W)
+    return s
+
+
+def make_bepepel_weights(cfg, seed: int = 0, device="cpu", scale: float = 1.0):
+    """Seeded random weights (bfloat16 torch tensors) with nothing at a value that would hide a dropped term: norm gains around 1,
+    non-zero biases, decay pre-activations that keep a gla state for tens of tokens, step sizes and decay rates of the state-space
+    heads spread over a decade, skip weights around 1."""
+    import torch
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    on_gpu = str(device) != "cpu"
+    gd = torch.Generator(device=device).manual_seed(seed) if on_gpu else g
+
+    def rnd(shape, big=False):
+        if big and on_gpu:
+            return torch.randn(shape, generator=gd, device=device, dtype=torch.float32)
+        return torch.randn(shape, generator=g, dtype=torch.float32).to(device)
+
+    out = {}
+    for name, shp in bepepel_weight_shapes(cfg).items():
+        leaf = name.rsplit(".", 1)[-1]
+        if name.endswith(".conv"):
+            w = rnd(shp) / (shp[-1] ** 0.5)
+        elif leaf in ("norm1", "norm2", "norm", "D"):
+            w = 1.0 + 0.1 * rnd(shp)
+        elif name.endswith("mix.a2.b"):
+            w = 2.0 + 0.5 * rnd(shp)
+        elif leaf == "dt_bias":
+            w = -1.5 + 0.7 * rnd(shp)
+        elif leaf == "A_log":
+            w = 0.6 * rnd(shp)
+        elif leaf == "b":
+            w = 0.1 * rnd(shp)
+        elif leaf == "embed":
+            w = rnd(shp, big=True)
+        else:
+            w = (scale / (shp[-1] ** 0.5)) * rnd(shp, big=True)
+        out[name] = w.to(torch.bfloat16)
+    return out
+
+
+def load_bepepel_safetensors(path: str, cfg):
+    """The tensors of ``<path>/model.safetensors`` by their own names, on the host, checked against the shapes the
+    configuration implies.  The low rank of a gla layer's decay projection is not in the configuration: it is read off
+    ``l{i}.mix.a1`` and written into ``cfg``."""
+    raw = read_checkpoint_dir(path)
+    for i, l in enumerate(cfg.layers):
+        if l.kind == "gla" and f"l{i}.mix.a1" in raw:
+            l.a_rank = int(raw[f"l{i}.mix.a1"].shape[0])
+    want = bepepel_weight_shapes(cfg)
+    missing = [k for k in want if k not in raw]
+    if missing:
+        raise KeyError(f"{path}: tensors missing for this configuration: {missing[:6]}{' ...' if len(missing) > 6 else ''}")
+    for k, shp in want.items():
+        if tuple(raw[k].shape) != tuple(shp):
+            raise ValueError(f"{path}: {k} has shape {tuple(raw[k].shape)}, the configuration implies {tuple(shp)}")
+    return {k: raw[k] for k in want}
