@@ -84,6 +84,37 @@ def rotate_pairs(x, positions, freqs):
     return out
 
 
+# ---- attention over explicit lists of visible keys ---------------------------------------------------------------------------------------
+def sees(i, j, window, keep_first):
+    """Does the query at position i see the key at position j?"""
+    return j <= i and (window <= 0 or i - j < window or j < keep_first)
+
+
+def softmax_over_seen(q, keys, vals, qpos, window, keep_first, scale):
+    """q [n, D] at positions qpos; keys [m, D] and vals [m, Dv] at positions 0 .. m - 1.  Returns [n, Dv]."""
+    out = torch.zeros(q.shape[0], vals.shape[1], dtype=F)
+    for t, i in enumerate(qpos):
+        seen = [j for j in range(keys.shape[0]) if sees(i, j, window, keep_first)]
+        w = torch.softmax((keys[seen] @ q[t]) * scale, dim=0)
+        out[t] = w @ vals[seen]
+    return out
+
+
+# ---- a matrix state with a decay per token -------------------------------------------------------------------------------------------------
+def matrix_state_steps(q, k, v, decay, S):
+    """S_t = diag(decay_t) S_(t-1) + k_t v_t^T, o_t = S_t^T q_t, token by token.  q, k [n, D]; v [n, Dv]; decay [n, D] (or [n, 1]: one
+    decay for all rows); S [D, Dv].  Returns the outputs [n, Dv] and the last state."""
+    out = torch.zeros(q.shape[0], v.shape[1], dtype=F)
+    for t in range(q.shape[0]):
+        S = decay[t].reshape(-1, 1) * S + k[t].reshape(-1, 1) * v[t].reshape(1, -1)
+        out[t] = S.T @ q[t]
+    return out, S
+
+
+def to_f64(weights):
+    return {k: v.to("cpu", F) for k, v in weights.items()}
+
+
 # ---- the mixers ----------------------------------------------------------------------------------------------------------------------
 def gla_mixer(h, p, pre, lay, eps, carry):
     """Gated linear attention with one decay per key channel and token."""
@@ -98,9 +129,9 @@ def gla_mixer(h, p, pre, lay, eps, carry):
     if S is None:
         S = torch.zeros(H, D, Dv, dtype=F)
     o = torch.zeros(n, H, Dv, dtype=F)
-    for t in range(n):
-        S = alpha[t].unsqueeze(-1) * S + k[t].unsqueeze(-1) * v[t].unsqueeze(-2)
-        o[t] = torch.einsum("hdv,hd->hv", S, q[t])
+    S = S.clone()
+    for hh in range(H):
+        o[:, hh], S[hh] = matrix_state_steps(q[:, hh], k[:, hh], v[:, hh], alpha[:, hh], S[hh])
     carry["S"] = S
     o = unit_rms(o, eps) * p[pre + "norm"]
     return (o.reshape(n, H * Dv) * silu(h @ p[pre + "g"].T)) @ p[pre + "o"].T
@@ -129,14 +160,9 @@ def window_attention(h, p, pre, a, eps, pos0, carry):
     vals = v if "v" not in carry else torch.cat([carry["v"], v], dim=0)
     carry["k"], carry["v"] = keys, vals
     out = torch.zeros(n, H, Dv, dtype=F)
-    for t in range(n):
-        i = pos0 + t
-        seen = [j for j in range(i + 1) if (a.window <= 0 or i - j < a.window or j < a.keep_first)]
-        for hh in range(H):
-            g = hh // (H // G)
-            s = torch.stack([(q[t, hh] * keys[j, g]).sum() * a.scale for j in seen])
-            w = torch.softmax(s, dim=0)
-            out[t, hh] = sum(w[x] * vals[j, g] for x, j in enumerate(seen))
+    for hh in range(H):
+        g = hh // (H // G)
+        out[:, hh] = softmax_over_seen(q[:, hh], keys[:, g], vals[:, g], list(range(pos0, pos0 + n)), a.window, a.keep_first, a.scale)
     return out.reshape(n, H * Dv) @ p[pre + "o"].T
 
 
@@ -162,11 +188,11 @@ def ssd_mixer(h, p, pre, b, eps, carry):
     if S is None:
         S = torch.zeros(H, N, P, dtype=F)
     y = torch.zeros(n, H, P, dtype=F)
-    for t in range(n):
-        for hh in range(H):
-            g = hh // (H // G)
-            S[hh] = torch.exp(-A[hh] * dt[t, hh]) * S[hh] + dt[t, hh] * Bm[t, g].unsqueeze(-1) * x[t, hh].unsqueeze(0)
-            y[t, hh] = S[hh].T @ Cm[t, g] + p[pre + "D"][hh] * x[t, hh]
+    S = S.clone()
+    for hh in range(H):
+        g = hh // (H // G)
+        y[:, hh], S[hh] = matrix_state_steps(Cm[:, g], Bm[:, g], dt[:, hh:hh + 1] * x[:, hh], torch.exp(-A[hh] * dt[:, hh:hh + 1]), S[hh])
+        y[:, hh] += p[pre + "D"][hh] * x[:, hh]
     carry["S"] = S
     y = y.reshape(n, inner) * silu(z)
     parts = b.norm_groups
@@ -228,3 +254,13 @@ def forward(cfg, p, tokens, pos0=0, carry=None, return_streams=False):
         streams.append(x)
     logits = layer_norm(x, p["final.norm"], p["final.norm.b"], eps) @ p["head"].T * cfg.logit_scale
     return (logits, torch.stack(streams)) if return_streams else logits
+
+
+def forward_in_portions(cfg, p, tokens, cuts):
+    """The same sequence fed in portions of the given sizes, each continuing from what the ones before left."""
+    carry = [{} for _ in cfg.layers]
+    out, at = [], 0
+    for c in cuts:
+        out.append(forward(cfg, p, tokens[at:at + c], pos0=at, carry=carry))
+        at += c
+    return torch.cat(out)
