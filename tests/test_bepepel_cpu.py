@@ -1,8 +1,10 @@
 """Bepepel without a GPU: the configuration reader and writer, the checkpoint reader, the registry, the host-side frequency table
 against the oracle's, and the float64 oracle (``oracle/bepepel_oracle.py``) against itself -- a prompt at once, token by token,
 and in portions must agree, which pins how it carries keys, convolution inputs and matrix states from step to step."""
+import ctypes
 import json
 import math
+import os
 
 import pytest
 import torch
@@ -150,3 +152,24 @@ def dataclass_with(s, **kw):
     for k, v in kw.items():
         setattr(s2, k, v)
     return s2
+
+
+def test_blocks_reject_bad_arguments_on_the_host():
+    """The library checks its arguments before it launches anything, so these calls need no GPU."""
+    from promptcache_amd import _blocks
+    assert os.path.exists(_blocks.lib_path()), "run __graft_entry__.build() first"
+    lb = _blocks.load(build_missing=False)
+    g = _blocks.GlaArgs(ctypes.sizeof(_blocks.GlaArgs), 0, None, None, None, 600, 600, 16, None, 600, 300, None, None, 0, None, 1, None, 10 ** 6,
+                        2, 2, 300, 8, 1.0, None, 16, None)
+    assert lb.pcb_gla(ctypes.byref(g), None) == -2001 and b"256 key columns" in lb.pcb_last_error_string()
+    g.dim, g.dcols = 64, 3                                    # a decay per key column, or one per head: nothing between
+    assert lb.pcb_gla(ctypes.byref(g), None) == -2001 and b"bad sizes" in lb.pcb_last_error_string()
+    g.dcols, g.Hk = 64, 3                                     # value heads must divide over the key heads
+    assert lb.pcb_gla(ctypes.byref(g), None) == -2001
+    g.Hk = 1
+    assert lb.pcb_gla(ctypes.byref(g), None) == -2001 and b"null pointer" in lb.pcb_last_error_string()
+    g.struct_bytes -= 8
+    assert lb.pcb_gla(ctypes.byref(g), None) == -2001 and b"struct size" in lb.pcb_last_error_string()
+    # a skip path without its weights
+    assert lb.pcb_gated_norm(None, 12, None, None, 0, None, 12, 0, 1e-6, 2, 12, 4, 1, 1, 12, None, 4, None) == -2001 and \
+        b"skip" in lb.pcb_last_error_string()

@@ -143,7 +143,7 @@ def test_blocks_reject_bad_arguments_on_the_host():
     h = _blocks.HeadPrepArgs(ctypes.sizeof(_blocks.HeadPrepArgs), 0, 0, 1, None, None, 1.0, 1e-6)
     h.seg[0] = _blocks.HeadPrepSeg(None, 8, 8, 1, 8, 0, None, None, None, 0, None, 0, 3, 4, None, 8, None, 8, 1)
     assert lb.pcb_head_prep(ctypes.byref(h), None) == -2001 and b"pairs" in lb.pcb_last_error_string()      # an odd first rotated column
-    assert lb.pcb_gated_norm(None, 12, None, None, 0, None, 12, 0, 1e-6, 2, 12, 5, None) == -2001 and b"divide" in lb.pcb_last_error_string()
+    assert lb.pcb_gated_norm(None, 12, None, None, 0, None, 12, 0, 1e-6, 2, 12, 5, 0, None, 0, None, 0, None) == -2001 and b"divide" in lb.pcb_last_error_string()
     assert lb.pcb_embed_scaled_rows(None, 0, None, 2.0, None, 3, 8, 10, None) == -2001 and b"null pointer" in lb.pcb_last_error_string()
 
 

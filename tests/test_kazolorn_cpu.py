@@ -175,7 +175,7 @@ def test_blocks_library_exports_what_the_header_declares():
         assert hasattr(lib, name), name
         assert len(_blocks.SIGNATURES[name][1]) == arity, name
     lb = _blocks.load(build_missing=False)
-    assert lb.pcb_version() == _blocks.ABI_VERSION == 3
+    assert lb.pcb_version() == _blocks.ABI_VERSION == 4
     assert lb.pcb_embed_rows(None, 0, None, None, 3, 8, 10, None) == -2001 and b"null pointer" in lb.pcb_last_error_string()
     assert lb.pcb_attn_talk_band(5, 100) == 32 and lb.pcb_attn_talk_band(0, 100) == 128 and lb.pcb_attn_talk_band(500, 100) == 128
 
