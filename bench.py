@@ -784,6 +784,46 @@ def run_fivesun(args):
     print(json.dumps(out))
 
 
+def run_bepepel(args):
+    """Throughput of the Bepepel stack beside the Dibizen stack (the closest existing model: the same building-block library, bf16
+    tensors, an fp32 residual, a decayed linear attention, a softmax attention, a selective scan and routed experts among its
+    parts) at equal width, heads and depth, with feed-forwards of about equal work (Dibizen: 2 of 16 two-matrix experts of width
+    w, 4 w^2 per token; Bepepel: 2 of 16 three-matrix experts of width w / 2 plus a shared one, 4.5 w^2).
+
+    Per size: one prompt of 2048 tokens (tokens/s of the prefill), then decoding at a context of 2048 with 1 and 8 requests.
+    `mixed` = gla, parallel, gla, gla; `gla` / `parallel` = four layers of that mixer alone, which is what prices each mixer's
+    kernels (beside Dibizen's `lightning`, and its `attention` and `mamba1`, whose work a parallel layer does side by side).  The
+    attention half sees a window of 1024 positions and keeps the first 4; the state-space half has width / 64 heads of 64 channels
+    with 128 states.  Random weights, synthetic tokens."""
+    import torch
+    import __graft_entry__ as ge
+    ge.build()
+    from promptcache_amd.model import Bepepel, Dibizen
+    from promptcache_amd.model.config import BepepelShape, DibizenShape
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    sizes = {"2k": dict(width=2048, heads=16, kv=4), "4k": dict(width=4096, heads=32, kv=8)}
+    L, V, T, steps, warm = 4, 32000, 2048, max(4, min(args.steps, 20)), max(1, min(args.warmup, 3))
+    g = torch.Generator().manual_seed(0)
+    out = {"metric": "bepepel_throughput", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "layers": L, "prompt": T, "sizes": {}}
+    patterns = {"mixed": ["gla", "parallel", "gla", "gla"], "gla": ["gla"] * L, "parallel": ["parallel"] * L}
+    for key in args.bepepel_sizes.split(","):
+        c = sizes[key]
+        w, h = c["width"], c["heads"]
+        row = {"width": w, "heads": h}
+        for pk in (("lightning", "attention", "mamba1") if args.bepepel_baseline else ()):
+            dz = DibizenShape.uniform(V, w, [pk] * L, h, c["kv"], w // h, 16, 2, w, streams=1, inner=2 * w, state=16, max_positions=T + 256,
+                                      name=f"dibizen-{key}-{pk}")
+            row["dibizen_" + pk] = slot_model_case(Dibizen(shape=dz, random_init=True, seed=0, device=dev), V, T, steps, warm, g)
+        for pk in args.bepepel_patterns.split(","):
+            shape = BepepelShape.uniform(V, w, patterns[pk], h, c["kv"], w // h, experts=16, top=2, expert_ff=w // 2, window=1024,
+                                         keep_first=4, name=f"bepepel-{key}-{pk}")
+            row["bepepel_" + pk] = slot_model_case(Bepepel(shape=shape, random_init=True, seed=0, device=dev), V, T, steps, warm, g)
+        out["sizes"][key] = row
+        print(json.dumps({key: row}), file=sys.stderr, flush=True)
+    print(json.dumps(out))
+
+
 def run_kazolorn(args):
     """Throughput of the Kazolorn stack beside the MPT stack at equal width, heads, depth and feed-forward width.
 
@@ -887,6 +927,12 @@ def main():
                          "real models (random weights), beside the Kazolorn stack (the closest existing model) at equal size")
     ap.add_argument("--dibizen-sizes", default="2k,4k", help="--dibizen: which sizes (2k, 4k)")
     ap.add_argument("--dibizen-patterns", default="mixed,attention,lightning,mamba1", help="--dibizen: which layer patterns")
+    ap.add_argument("--bepepel", action="store_true",
+                    help="instead of the default workload: prefill / decode throughput of the Bepepel design at layer sizes of "
+                         "real models, beside the Dibizen stack at equal size")
+    ap.add_argument("--bepepel-sizes", default="2k,4k", help="--bepepel: which sizes (2k, 4k)")
+    ap.add_argument("--bepepel-patterns", default="mixed,gla,parallel", help="--bepepel: which layer patterns")
+    ap.add_argument("--bepepel-baseline", type=int, default=1, help="--bepepel: 0 leaves the Dibizen stacks out (kernel profiles of Bepepel alone)")
     ap.add_argument("--fivesun", action="store_true",
                     help="instead of the default workload: prefill / decode throughput of the Fivesun design at layer sizes of "
                          "real models (random weights), beside the Dibizen stack (the closest existing model) at equal size")
@@ -902,6 +948,9 @@ def main():
         return
     if args.dibizen:
         run_dibizen(args)
+        return
+    if args.bepepel:
+        run_bepepel(args)
         return
     if args.fivesun:
         run_fivesun(args)

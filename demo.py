@@ -10,6 +10,7 @@ cache and once with ``no_cache=True``, printing the two timed intervals of each 
                                                      # plain generation, single and batched (no prompt modules for this design)
     python demo.py --model dibizen                   # the Dibizen design (lightning / attention / mamba1 layers), likewise
     python demo.py --model fivesun                   # the Fivesun design (attention / latent attention / mlstm layers), likewise
+    python demo.py --model bepepel                   # the Bepepel design (gla / parallel attention + state-space layers), likewise
 
 There is no network on the build / bench machines, so without a checkpoint directory the adapters use seeded random
 weights at the named shape and the deterministic stand-in tokenizer: the text is noise, the timings are real.
@@ -22,8 +23,8 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(ROOT, "prompt-cache_amd"))
 
 from promptcache_amd import CacheEngine, GenerationEngine, GenerationParameters, Prompt, read_file, synth  # noqa: E402
-from promptcache_amd.model import CodeLlama, Dibizen, Falcon, Fivesun, Kazolorn, Llama2, Mpt, load_language_model  # noqa: E402
-from promptcache_amd.model.config import DibizenShape, FivesunShape, KazolornShape  # noqa: E402
+from promptcache_amd.model import Bepepel, CodeLlama, Dibizen, Falcon, Fivesun, Kazolorn, Llama2, Mpt, load_language_model  # noqa: E402
+from promptcache_amd.model.config import BepepelShape, DibizenShape, FivesunShape, KazolornShape  # noqa: E402
 
 ADAPTERS = {"llama": (Llama2, "llama2-7b"), "codellama": (CodeLlama, "codellama-7b"), "falcon": (Falcon, "falcon-7b"),
             "mpt": (Mpt, "mpt-7b")}
@@ -51,7 +52,7 @@ def kazolorn_demo(lm, a):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--model", default="llama", help="llama | codellama | falcon | mpt | kazolorn | dibizen | fivesun | <checkpoint directory>")
+    ap.add_argument("--model", default="llama", help="llama | codellama | falcon | mpt | kazolorn | dibizen | fivesun | bepepel | <checkpoint directory>")
     ap.add_argument("--schema", help="PML schema file (default: a synthetic game-like schema, 7 modules)")
     ap.add_argument("--prompt-file", help="PML prompt file referencing the schema")
     ap.add_argument("--max-ctx", type=int, default=5000)
@@ -71,10 +72,13 @@ def main():
     elif a.model == "fivesun":
         lm = Fivesun(shape=FivesunShape.uniform(32000, 1024, ["attention", "latent_attention", "attention", "mlstm"], 8, 2, 128, 2048,
                                                 chunk=1024, window=512, kv_rank=192, rot_dim=64), random_init=True)
+    elif a.model == "bepepel":
+        lm = Bepepel(shape=BepepelShape.uniform(32000, 1024, ["gla", "parallel", "gla", "gla"], 8, 2, 128, experts=8, top=2, expert_ff=512,
+                                                window=512, keep_first=4), random_init=True)
     else:
         cls, shape = ADAPTERS[a.model]
         lm = cls(shape, random_init=True)
-    if isinstance(lm, (Kazolorn, Dibizen, Fivesun)):
+    if isinstance(lm, (Kazolorn, Dibizen, Fivesun, Bepepel)):
         kazolorn_demo(lm, a)
         return
     preproc = [lm.get_formatter()]

@@ -339,7 +339,9 @@ template <typename E>
 int dispatch(const pcb_linear_args& a, hipStream_t stream) {
     // rows per group decide the row tile: many rows -> 128-row panels, few -> 32-row panels (the weights stream once)
     const int rows = a.n_groups > 0 ? pcb_ceil_div(a.M, a.n_groups) : a.M;
-    const bool big = rows > 64;
+    // (a narrow result -- router logits, step sizes: N <= 64 -- takes the 32-row panels too: 128-row panels would leave M / 128
+    // workgroups on the chip, each walking all of K)
+    const bool big = rows > 64 && a.N > 64;
     if (rows <= 16) {
         const dim3 grid(pcb_ceil_div(a.N, 16), pcb_ceil_div(a.M, 16) + (a.n_groups > 0 ? a.n_groups : 0));
         switch (a.epilogue) {

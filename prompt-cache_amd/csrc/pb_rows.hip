@@ -388,16 +388,19 @@ __global__ __launch_bounds__(256) void gated_norm_kernel(const float* __restrict
     }
 }
 
-// the same with a norm per run of `group` columns (a head): one wave per (row, group) pair, four pairs per workgroup.  A skip path
-// (x + skip_w[c / skip_group] * skip) and a gate that comes before the norm are this kernel's alone.
-template <typename E>
+// the same with a norm per run of `group` columns (a head): one wave per (row, group) pair, four pairs per workgroup -- or, WIDE, a
+// whole workgroup per pair (groups of hundreds of columns, where one wave's chain of dependent loads would be the launch's length).
+// A skip path (x + skip_w[c / skip_group] * skip) and a gate that comes before the norm are this kernel's alone.
+template <typename E, bool WIDE>
 __global__ __launch_bounds__(256) void gated_group_norm_kernel(const float* __restrict__ x, int64_t ldx, const float* __restrict__ gain,
                                                                const E* __restrict__ gate, int64_t ldg, E* __restrict__ out, int64_t ldo,
                                                                float eps, int cols, int group, int64_t n_pairs, int gate_first,
                                                                const E* __restrict__ skip, int64_t lds, const float* __restrict__ skip_w,
                                                                int skip_group) {
-    const int lane = threadIdx.x & 63;
-    const int64_t pair = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    __shared__ float red[16];
+    constexpr int TPP = WIDE ? 256 : 64;                   // threads per pair
+    const int lane = WIDE ? (int)threadIdx.x : (int)(threadIdx.x & 63);
+    const int64_t pair = WIDE ? (int64_t)blockIdx.x : (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (pair >= n_pairs) return;
     const int per = cols / group;
     const int64_t r = pair / per;
@@ -408,14 +411,17 @@ __global__ __launch_bounds__(256) void gated_group_norm_kernel(const float* __re
         if (gate_first && gate) v *= to_f32(gate[r * ldg + c]);
         return v;
     };
-    float ss = 0.0f;
-    for (int c = lane; c < group; c += 64) {
+    float ss[1] = {0.0f};
+    for (int c = lane; c < group; c += TPP) {
         const float v = value(c0 + c);
-        ss += v * v;
+        ss[0] += v * v;
     }
-    ss = wave_sum(ss);
-    const float inv = 1.0f / sqrtf(ss / (float)group + eps);
-    for (int c = lane; c < group; c += 64) {
+    if (WIDE)
+        block_sum<1>(ss, red);
+    else
+        ss[0] = wave_sum(ss[0]);
+    const float inv = 1.0f / sqrtf(ss[0] / (float)group + eps);
+    for (int c = lane; c < group; c += TPP) {
         float v = value(c0 + c) * inv;
         if (gain) v *= gain[c0 + c];
         if (gate && !gate_first) v *= to_f32(gate[r * ldg + c0 + c]);
@@ -641,13 +647,17 @@ PCB_EXPORT int pcb_gated_norm(const float* x, int64_t ldx, const float* gain, co
     if (gate_first || skip) group_cols = group_cols > 0 ? group_cols : cols;       // (the per-group kernel knows these two)
     if ((group_cols > 0 && group_cols < cols) || gate_first || skip) {
         const int64_t pairs = (int64_t)n_rows * (cols / group_cols);
-        const dim3 grid((unsigned)((pairs + 3) / 4));
-        if (dtype == PCB_BF16)
-            hipLaunchKernelGGL(gated_group_norm_kernel<bf16_t>, grid, dim3(256), 0, (hipStream_t)stream, x, ldx, gain, (const bf16_t*)gate,
-                               ldg, (bf16_t*)out, ldo, eps, cols, group_cols, pairs, gate_first, (const bf16_t*)skip, lds, skip_w, skip_group);
-        else
-            hipLaunchKernelGGL(gated_group_norm_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, x, ldx, gain, (const float*)gate,
-                               ldg, (float*)out, ldo, eps, cols, group_cols, pairs, gate_first, (const float*)skip, lds, skip_w, skip_group);
+        const bool wide = group_cols >= 512;
+        const dim3 grid((unsigned)(wide ? pairs : (pairs + 3) / 4));
+#define PCB_GGN(E_, WIDE_)                                                                                                                 \
+    hipLaunchKernelGGL((gated_group_norm_kernel<E_, WIDE_>), grid, dim3(256), 0, (hipStream_t)stream, x, ldx, gain, (const E_*)gate, ldg, \
+                       (E_*)out, ldo, eps, cols, group_cols, pairs, gate_first, (const E_*)skip, lds, skip_w, skip_group)
+        if (dtype == PCB_BF16) {
+            if (wide) PCB_GGN(bf16_t, true); else PCB_GGN(bf16_t, false);
+        } else {
+            if (wide) PCB_GGN(float, true); else PCB_GGN(float, false);
+        }
+#undef PCB_GGN
         return pcb_check_launch("gated_group_norm_kernel");
     }
     if (dtype == PCB_BF16)

@@ -18,10 +18,11 @@ With the residual x in fp32, m = ``residual_mult`` and ln(.) a layer norm with w
                 projection's epilogue; per head S <- diag(decay) S + k v^T, o = S^T q / sqrt(dim) (pcb_gla); y = Wo (rms(o) gain * g)
     parallel    left:  q | k | v of ONE projection with biases -> causal convolution (pcb_causal_conv) -> per head unit RMS and rotary
                        pairs; k rows and v columns land in the slot's cache (pcb_head_prep); softmax over a sliding window that keeps
-                       the first positions (pcb_attn_softmax); y = left_scale * Wo (.)
+                       the first positions (pcb_attn_softmax); y = Wo (.)
                 right: z | x | B | C of ONE projection (SiLU on z), dt = softplus(W_dt h + b) in fp32; x | B | C through a causal
                        convolution and SiLU; per head S <- exp(-e^A_log dt) S + dt B x^T, y = S^T C (pcb_gla with one decay per head);
-                       rms_parts((y + D x) silu(z)) gain (pcb_gated_norm, the gate first); y += right_scale * Wo (.)
+                       rms_parts((y + D x) silu(z)) gain (pcb_gated_norm, the gate first); y += right_scale / left_scale * Wo (.),
+                       and the residual step multiplies y by left_scale
     dense       Wdown (gelu_tanh(Wgate h) * Wup h), the product in the first projection's epilogue
     experts     router logits (fp32, with bias) -> the top logits and the softmax over them (pcb_router_select); pairs bucketed by
                 expert (pcb_moe_plan); silu(Wgate h) * Wup h and Wdown per bucket (grouped pcb_linear); y = sum_k w_k (expert result)
@@ -125,7 +126,7 @@ class BepepelHIP(SlotModel):
                     r_in=w_in[:nm].contiguous(), r_dt=w_in[nm:].contiguous(), r_dt_b=e(rp + "dt_bias"),
                     r_conv=e(rp + "conv") if b.conv else None, r_conv_b=e(rp + "conv.b") if b.conv else None,
                     r_rate=(-torch.exp(f(rp + "A_log"))).contiguous(), r_D=f(rp + "D"), r_gain=f(rp + "norm"), r_wo=e(rp + "o"),
-                    r_scale=const(W, l.right_scale), chain_coef=const(b.heads * b.state * b.vdim, 1.0))
+                    r_scale=const(W, l.right_scale / l.left_scale if l.left_scale != 0.0 else l.right_scale), chain_coef=const(b.heads * b.state * b.vdim, 1.0))
             if l.ff_kind:
                 q = p + "mlp."
                 ent.update(norm2=(f(p + "norm2"), f(p + "norm2.b")))
@@ -289,8 +290,8 @@ class BepepelHIP(SlotModel):
 
         def step(norm, out, **kw):
             nonlocal pending
-            B.post_norm(x, gain=norm[0], bias=norm[1], layer_norm=True, out=out, eps=eps, y_scale=mult, n_rows=kw.pop("n_rows", T),
-                        **pending, **kw)
+            B.post_norm(x, gain=norm[0], bias=norm[1], layer_norm=True, out=out, eps=eps, n_rows=kw.pop("n_rows", T),
+                        **{"y_scale": mult, **pending}, **kw)
             pending = {}
 
         for i, lw in enumerate(layers):
@@ -298,9 +299,9 @@ class BepepelHIP(SlotModel):
             step(lw["norm1"], h)
             if l.kind == "gla":
                 self._gla(arena, i, l, lw, h, y1, tb, T, R)
+                pending = dict(y=y1)
             else:
-                self._parallel(arena, i, l, lw, h, y1, tb, T, R, d["n_tiles"])
-            pending = dict(y=y1)
+                pending = dict(y=y1, y_scale=mult * self._parallel(arena, i, l, lw, h, y1, tb, T, R, d["n_tiles"]))
             if l.ff_kind:
                 step(lw["norm2"], h)
                 if l.ff_kind == "dense":
@@ -309,7 +310,7 @@ class BepepelHIP(SlotModel):
                     self._experts(l, lw, h, y2, T)
                 pending = dict(y=y2)
             if streams is not None:
-                B.post_norm(x, eps=eps, n_rows=T, x_out=streams[i], y_scale=mult, **pending)
+                B.post_norm(x, eps=eps, n_rows=T, x_out=streams[i], **{"y_scale": mult, **pending})
                 pending = {}
         if d["n_want"]:
             nw = d["n_want"]
@@ -356,6 +357,9 @@ class BepepelHIP(SlotModel):
         return 1 if n_tiles * heads >= 512 or arena.cap <= 256 else max(1, min(16, 1024 // (n_tiles * heads), arena.cap // 128))
 
     def _parallel(self, arena, i, l, lw, h, y, tb, T, R, n_tiles):
+        """Leaves left + (right_scale / left_scale) right in y and returns left_scale, the factor that is still to come (the
+        residual step multiplies by it together with the residual factor): the plain store of the left projection is the faster
+        epilogue.  A left_scale of 0 is applied in the projection itself."""
         E, f32, eps = self.dtype, torch.float32, self.config.norm_eps
         a, b = l.left, l.right
         states = list(arena.states[i])
@@ -390,7 +394,10 @@ class BepepelHIP(SlotModel):
         B.attn_softmax(q, HD, tb["tiles"], n_tiles, plane, (arena.slot_stride(i), arena.head_stride(i), D), vplane, 0,
                        (arena.col_slot_stride(i), arena.col_head_stride(i), arena.cap), True, H, G, D, Dv, a.scale, att,
                        window=a.window, keep_first=a.keep_first, n_splits=splits, part=part)
-        B.linear(att, lw["l_wo"], y, M=T, act=B.ACT_SCALE, act_param=lw["l_scale"])
+        if lw["l_scale"] != 0.0:
+            B.linear(att, lw["l_wo"], y, M=T)
+        else:
+            B.linear(att, lw["l_wo"], y, M=T, act=B.ACT_SCALE, act_param=0.0)
         # ---- right: the state-space half
         Hs, Pv, N, Gs = b.heads, b.vdim, b.state, b.groups
         inner, CC = b.inner, b.conv_channels
@@ -416,6 +423,7 @@ class BepepelHIP(SlotModel):
         B.gated_norm(ys, lw["r_gain"], Z, NR, yn, eps, T, group=inner // b.norm_groups, gate_first=True, skip=xbc, lds=ldx,
                      skip_w=lw["r_D"], skip_group=Pv)
         B.linear(yn, lw["r_wo"], y, M=T, epilogue=B.EPI_SCALE_ADD, col_scale=lw["r_scale"])
+        return lw["l_scale"] if lw["l_scale"] != 0.0 else 1.0
 
     # ---- feed-forwards -----------------------------------------------------------------------------------------------------------------
     def _unit(self, u, h, y, T, act, add=False):
