@@ -202,6 +202,78 @@ def test_log_decay_and_scaled_epilogues(dtype):
     assert rel(y, -2.5 * (f64(x[:, 3:]) @ f64(w).T)) < 1e-5
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("taps,bias,act", [(3, False, False), (4, True, True), (2, False, True), (1, False, False), (1, True, True), (7, True, False)])
+def test_short_convolution_over_steps_and_reused_slots(dtype, taps, bias, act):
+    """Two sequences on two slots, fed in portions of unequal sizes (also of one token, also shorter than the taps reach back); a
+    slot that held another sequence starts from zeros when its new sequence starts at position 0."""
+    Cn, ld = 37, 45
+    w = rnd(Cn, taps, dtype=dtype, seed=1)
+    b = rnd(Cn, dtype=dtype, seed=2) if bias else None
+    state = torch.full((2, taps - 1, Cn), 9.0, dtype=dtype, device=DEV)               # (what a slot held before must not matter)
+    seqs = {0: rnd(23, ld, dtype=dtype, seed=3), 1: rnd(11, ld, dtype=dtype, seed=4)}
+    plan = [{0: 1, 1: 4}, {0: 2, 1: 1}, {0: 9}, {1: 6, 0: 11}]                         # tokens per slot and step
+    at, got = {0: 0, 1: 0}, {0: [], 1: []}
+    for step in plan:
+        rows, meta, reqs = [], [], []
+        for slot, n in step.items():
+            reqs.append((slot, at[slot], n, len(meta)))
+            meta += [(slot, at[slot] + i, i, 0) for i in range(n)]
+            rows.append(seqs[slot][at[slot]:at[slot] + n])
+        x = torch.cat(rows).contiguous()
+        out = torch.empty(len(meta), Cn, dtype=dtype, device=DEV)
+        B().causal_conv(x[:, 5:], ld, w, b, act, dev_i32(meta), state, out, len(meta))
+        if taps > 1:
+            B().conv_state_update(x[:, 5:], ld, dev_i32(reqs), len(reqs), state)
+        r = 0
+        for slot, n in step.items():
+            got[slot].append(out[r:r + n])
+            at[slot] += n
+            r += n
+    for slot in (0, 1):
+        want, _ = O.short_conv(f64(seqs[slot][:, 5:5 + Cn]), f64(w), f64(b) if bias else None, torch.zeros(taps - 1, Cn, dtype=F64))
+        if act:
+            want = O.silu(want)
+        assert rel(torch.cat(got[slot]), want) < tol(dtype, 1e-6, 6e-3)
+    # slot 1 goes to a new sequence: position 0 again
+    x = rnd(5, ld, dtype=dtype, seed=8)
+    out = torch.empty(5, Cn, dtype=dtype, device=DEV)
+    B().causal_conv(x[:, 5:], ld, w, b, act, dev_i32([(1, i, i, 0) for i in range(5)]), state, out, 5)
+    want, _ = O.short_conv(f64(x[:, 5:5 + Cn]), f64(w), f64(b) if bias else None, torch.zeros(taps - 1, Cn, dtype=F64))
+    assert rel(out, O.silu(want) if act else want) < tol(dtype, 1e-6, 6e-3)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("D,rot,scaling", [(24, 16, (8.0, 1.0, 4.0, 64.0)), (10, 10, None), (64, 2, (4.0, 0.5, 2.0, 16.0)), (6, 0, None)])
+def test_rotation_then_unit_norm_per_head(dtype, D, rot, scaling):
+    """The design rotates the leading pairs and THEN divides each head by its root mean square; the kernel divides first.  Both are
+    checked against the oracle's order, at positions from 0 to the thousands, with plain and wavelength-scaled frequencies."""
+    from promptcache_amd.model.bepepel_hip import scaled_rotary_frequencies
+    H, n = 3, 40
+    x = rnd(n, H * D + 7, dtype=dtype, seed=1, scale=3.0)
+    pos = torch.tensor([0, 1, 2, 3, 63, 64, 65, 511, 512, 1000] + list(range(2000, 2030)), dtype=torch.int32, device=DEV)
+    out = torch.empty(n, H * D, dtype=dtype, device=DEV)
+    freqs = torch.from_numpy(scaled_rotary_frequencies(777.0, rot, scaling)).to(DEV) if rot else None
+    B().head_prep([B().head_seg(x[:, 7:], H * D + 7, H, D, out, norm=True, rot_dims=rot, ld_dst=H * D)], n, dtype, pos=pos, freqs=freqs, eps=1e-5)
+    fr = O.rotary_frequencies(777.0, rot, scaling) if rot else torch.zeros(0, dtype=F64)
+    want = O.unit_rms(O.rotate_pairs(f64(x[:, 7:]).view(n, H, D), pos.cpu(), fr), 1e-5).reshape(n, H * D)
+    assert rel(out, want) < tol(dtype, 2e-6, 4e-3)
+
+
+@pytest.mark.parametrize("n_exp,top", [(16, 4), (5, 5), (1, 1), (9, 1), (64, 8)])
+def test_router_takes_the_top_logits_and_the_softmax_over_them(n_exp, top):
+    T, K = 50, 24
+    h, wr, br = rnd(T, K, seed=1), rnd(n_exp, K, seed=2), rnd(n_exp, seed=3, scale=2.0)
+    logits = torch.empty(T, n_exp, dtype=torch.float32, device=DEV)
+    B().linear(h, wr, logits, M=T, bias=br)
+    expert = torch.empty(T * top, dtype=torch.int32, device=DEV)
+    weight = torch.empty(T * top, dtype=torch.float32, device=DEV)
+    B().router_select(logits, top, expert, weight, T, score_fn=B().SCORE_SOFTMAX, renorm=True)
+    idx, w = O.route(f64(h), {"r.router": f64(wr), "r.router.b": f64(br)}, "r.", top)
+    assert torch.equal(expert.view(T, top).cpu().long(), idx) and rel(weight.view(T, top), w) < 1e-5
+    assert float((weight.view(T, top).sum(dim=1) - 1.0).abs().max()) < 1e-5
+
+
 def _recurrence_inputs(dtype, n, H, Hk, D, Dv, dcols, seed):
     q, k, v = rnd(n, Hk * D + 3, dtype=dtype, seed=seed), rnd(n, Hk * D + 5, dtype=dtype, seed=seed + 1), rnd(n, H * Dv, dtype=dtype, seed=seed + 2)
     ld = torch.rand(n, H * dcols, generator=torch.Generator().manual_seed(seed + 3)).to(DEV) * 0.5     # (times a negative rate: a log decay)
