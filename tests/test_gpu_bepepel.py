@@ -64,7 +64,7 @@ def gla(heads, dim, vdim, tau=6.0, rank=5, **ff):
 
 
 def par(H, G, D, Dv, window, keep, sh, sp, sn, sg=1, parts=1, convl=3, convr=4, rot=None, scaling=(4.0, 1.0, 4.0, 64.0), scale=None,
-        ls=1.2, rs=0.8, base=5000.0, **ff):
+        ls=1.25, rs=0.8, base=5000.0, **ff):
     left = BepepelAttention(heads=H, kv_heads=G, dim=D, vdim=Dv, scale=scale or 2.0 * D ** -0.5, conv=convl, window=window, keep_first=keep,
                             rot_base=base, rot_dims=D if rot is None else rot, rot_scaling=scaling)
     right = BepepelSSD(heads=sh, vdim=sp, state=sn, groups=sg, norm_groups=parts, conv=convr)
@@ -99,11 +99,11 @@ def shape_odd():
 
 def shape_wide():
     """Enough heads and columns to reach the wider kernel instantiations; windows longer than a key block, many kept tokens."""
-    return BepepelShape(vocab_size=320, hidden_size=128, norm_eps=1e-6, residual_mult=0.3, logit_scale=2.0, layers=[
+    return BepepelShape(vocab_size=320, hidden_size=128, norm_eps=1e-6, residual_mult=0.35, logit_scale=2.5, layers=[
         gla(2, 200, 136, tau=16.0, rank=16, **DENSE),
         par(8, 2, 128, 72, 64, 40, 4, 64, 128, sg=2, parts=2, rot=64, **MOE),
         gla(4, 64, 64, tau=8.0, rank=8),
-        par(4, 4, 272, 72, 100, 4, 10, 40, 100, sg=5, parts=5, convl=4, convr=3, rot=32, scaling=(8.0, 1.0, 4.0, 512.0), **DENSE),
+        par(4, 4, 272, 72, 100, 4, 10, 40, 100, sg=5, parts=5, convl=4, convr=3, rot=32, scaling=(6.0, 1.0, 4.0, 400.0), **DENSE),
     ])
 
 
@@ -551,10 +551,10 @@ def random_shape(rng):
             layers.append(par(G * rng.choice([1, 2, 3]), G, D, rng.choice([16, 40, 64, 128]), rng.choice([0, 1, 7, 32, 50, 100]), rng.choice([0, 1, 4, 40]),
                               sh, sp, rng.choice([4, 16, 48, 128]), sg=sg, parts=parts, convl=rng.choice([0, 2, 3, 4]), convr=rng.choice([0, 2, 4]),
                               rot=rng.choice([D, D // 4 * 2, 0]), scaling=rng.choice([None, (8.0, 1.0, 4.0, 128.0), (2.0, 0.5, 8.0, 32.0)]),
-                              scale=rng.choice([0.125, 0.5, 1.0]), ls=rng.choice([1.0, 1.2]), rs=rng.choice([1.0, 0.9]),
-                              base=rng.choice([250000.0, 1000.0]), **ff))
+                              scale=rng.choice([0.125, 0.5, 1.0]), ls=rng.choice([1.0, 1.3]), rs=rng.choice([1.0, 0.7]),
+                              base=rng.choice([300000.0, 1000.0]), **ff))
     return BepepelShape(vocab_size=rng.randrange(50, 900), hidden_size=width, norm_eps=rng.choice([1e-5, 1e-6]),
-                        residual_mult=rng.choice([1.0, 0.3]), logit_scale=rng.choice([1.0, 2.0]), layers=layers)
+                        residual_mult=rng.choice([1.0, 0.45]), logit_scale=rng.choice([1.0, 1.75]), layers=layers)
 
 
 @pytest.mark.parametrize("seed", range(8))
